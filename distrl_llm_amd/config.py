@@ -90,3 +90,10 @@ class EngineConfig:
     # the decode step (existing kernels only); LRU-evicted under pool
     # pressure. Off by default: RL rollouts use unique prompts.
     enable_prefix_caching: bool = False
+    # Layer-list (hybrid) models: number of per-sequence state slots
+    # (convolution tails, recurrent state); it bounds the live sequences.
+    # 0 = min(max_num_seqs, 256).
+    num_state_slots: int = 0
+    # Hybrid models: most tokens one step carries (decode tokens first,
+    # prompt portions fill the rest).
+    step_token_budget: int = 8192

@@ -1,0 +1,372 @@
+"""Generation engine for layer-list (hybrid) models.
+
+One step function runs a flat batch that mixes portions of prompts with
+single decode tokens: every row continues its sequence from the pages and
+state slot earlier steps left, however the prompt was cut. ``generate``
+is a continuous-batching scheduler over that step (decode tokens first,
+prompt portions fill the step's token budget; n-candidate fan-out forks
+the prompt's pages and state), with the same call signature as the dense
+:class:`Engine`, so the batcher, the server and the command line drive
+either. A trace replay (``bin/trace_run``) calls the same step directly.
+
+Numerics: the residual stream, norms, convolution, rotary angles,
+attention scores/softmax, recurrent state, router and the gated residual
+sum are fp32; matrix products run in the model dtype with fp32
+accumulation (true fp32 when the model dtype is fp32).
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence as Seq, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from ..config import EngineConfig, SamplingParams
+from ..models.hybrid import HybridLM, LatentAttentionSpec
+from ..ops import functional as OF
+from ..ops import seqmix as SM
+from ..utils.trace import trace_range
+from .kvcache import Sequence
+from .seqstate import LatentCachePool, StateSlotPool
+
+
+class HybridEngine:
+    def __init__(self, model: HybridLM, cfg: EngineConfig,
+                 device: Optional[torch.device] = None, seed: int = 0):
+        self.model = model
+        self.cfg = cfg
+        self.spec = model.spec
+        self.device = device if device is not None else model.device
+        self.dtype = model.dtype_
+        self._seq_counter = 0
+        self.generator = torch.Generator(device=self.device)
+        self.generator.manual_seed(seed)
+
+        num_slots = cfg.num_state_slots or min(cfg.max_num_seqs, 256)
+        num_blocks = cfg.num_kv_blocks
+        if num_blocks <= 0:
+            num_blocks = self._derive_num_blocks(num_slots)
+        self.pool = LatentCachePool(self.spec, num_blocks, cfg.kv_block_size,
+                                    self.dtype, self.device)
+        self.slots = StateSlotPool(self.spec, num_slots, self.device)
+
+    def _derive_num_blocks(self, num_slots: int) -> int:
+        bs = self.cfg.kv_block_size
+        per_block = LatentCachePool.bytes_per_block(self.spec, bs, self.dtype)
+        if self.device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(self.device)
+            budget = int(free * self.cfg.gpu_memory_utilization)
+        else:
+            budget = 64 * 1024 * 1024
+        n = max(budget // per_block, 16)
+        most = num_slots * LatentCachePool.blocks_for(self.cfg.max_seq_length, bs)
+        return int(min(n, most))
+
+    # ------------------------------------------------- sequence lifecycle
+
+    def open_sequence(self, prompt_ids: Seq[int] = (), parent_prompt: int = 0
+                      ) -> Sequence:
+        """Admit a sequence: it gets a zeroed state slot; pages are taken
+        as its tokens arrive."""
+        self._seq_counter += 1
+        q = Sequence(self._seq_counter, list(prompt_ids), parent_prompt)
+        q.slot = self.slots.alloc()
+        return q
+
+    def close_sequence(self, q: Sequence) -> None:
+        """Give a sequence's pages and slot back."""
+        q.finished = True
+        for b in q.block_table:
+            self.pool.allocator.free(b)
+        q.block_table = []
+        if q.slot is not None:
+            self.slots.free(q.slot)
+            q.slot = None
+
+    def fork_sequence(self, parent: Sequence) -> Sequence:
+        """A new sequence continuing from the parent's state: full pages
+        are shared by refcount, a partial last page and the state slot are
+        copied."""
+        bs = self.pool.block_size
+        child = self.open_sequence(parent.prompt_ids, parent.parent_prompt)
+        full = parent.context_len // bs
+        for b in parent.block_table[:full]:
+            self.pool.allocator.incref(b)
+            child.block_table.append(b)
+        if parent.context_len % bs:
+            nb = self.pool.allocator.alloc()
+            self.pool.copy_block(parent.block_table[full], nb)
+            child.block_table.append(nb)
+        self.slots.copy(parent.slot, child.slot)
+        child.context_len = parent.context_len
+        return child
+
+    def reset(self) -> None:
+        self.pool.allocator.reset()
+        self.slots.reset()
+
+    # --------------------------------------------------------------- step
+
+    @torch.no_grad()
+    def step(self, work: List[Tuple[Sequence, Seq[int]]],
+             want: Optional[List[Seq[int]]] = None,
+             capture: Optional[list] = None) -> torch.Tensor:
+        """Run the next tokens of every listed sequence as one flat batch.
+
+        work: (sequence, its next tokens) rows, each with >= 1 token.
+        want: per row, the places among its tokens whose logits are
+        returned (default: the last one). Returns fp32 [sum(want), vocab]
+        in row order. ``capture`` (a list) receives the residual stream
+        after every layer."""
+        bs = self.pool.block_size
+        dev = self.device
+        tokens, positions, tok_seq, page_slot, cu = [], [], [], [], [0]
+        slot_idx, want_rows = [], []
+        for b, (q, toks) in enumerate(work):
+            n = len(toks)
+            if n < 1:
+                raise ValueError("every row of a step needs at least one token")
+            p0 = q.context_len
+            need = LatentCachePool.blocks_for(p0 + n, bs)
+            while len(q.block_table) < need:
+                q.block_table.append(self.pool.allocator.alloc())
+            base = cu[-1]
+            for k in range(n):
+                p = p0 + k
+                positions.append(p)
+                page_slot.append(q.block_table[p // bs] * bs + p % bs)
+            tokens.extend(int(t) for t in toks)
+            tok_seq.extend([b] * n)
+            cu.append(base + n)
+            slot_idx.append(q.slot)
+            for w in ([n - 1] if want is None else want[b]):
+                if not 0 <= w < n:
+                    raise ValueError("wanted place outside the row's tokens")
+                want_rows.append(base + w)
+        max_nb = max(len(q.block_table) for q, _ in work)
+        tables = [q.block_table + [0] * (max_nb - len(q.block_table))
+                  for q, _ in work]
+
+        def i32(v):
+            return torch.tensor(v, dtype=torch.int32, device=dev)
+
+        meta = dict(positions=i32(positions), tok_seq=i32(tok_seq),
+                    page_slot=i32(page_slot), cu=i32(cu), slots=i32(slot_idx),
+                    block_tables=i32(tables))
+        logits = self._forward(torch.tensor(tokens, dtype=torch.long, device=dev),
+                               meta, torch.tensor(want_rows, dtype=torch.long,
+                                                  device=dev), capture)
+        for q, toks in work:
+            q.context_len += len(toks)
+        return logits
+
+    def _forward(self, tokens, meta, want_rows, capture=None) -> torch.Tensor:
+        S, M, dt = self.spec, self.model, self.dtype
+        eps, mult = S.norm_eps, S.residual_mult
+        T = tokens.shape[0]
+        pos, cu, slots = meta["positions"], meta["cu"], meta["slots"]
+        bs = self.pool.block_size
+
+        x, _ = SM.offset_rmsnorm(M.embed[tokens], M.embed_norm_w, eps, dt)
+        h32, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt)
+        last = S.num_layers - 1
+        for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
+            hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i], cu,
+                                    slots, dt)
+            gates = F.linear(hb, L.gate_w)
+            m = ls.mixer
+            if isinstance(m, LatentAttentionSpec):
+                own = m.kv_from is None
+                proj = F.linear(hm, L.in_w)
+                cache = self.pool.layer_rows(S, i)
+                q_rot = SM.latent_prepare(
+                    proj, m.heads, m.dim, m.rot_dim, m.kv_rank, own,
+                    L.latent_norm_w if own else None, eps, pos, m.rope_base,
+                    m.rope_dims, meta["page_slot"], cache)
+                q_nope = proj[:, :m.q_size].view(T, m.heads, m.dim + m.rot_dim)
+                q_lat = torch.bmm(q_nope[..., :m.dim].transpose(0, 1), L.uk)
+                o_lat = SM.latent_window_attention(
+                    q_lat, q_rot, cache, m.kv_rank, meta["block_tables"], bs,
+                    cu, meta["tok_seq"], pos, m.window, m.scale, dt)
+                v = torch.bmm(o_lat, L.uv.transpose(1, 2))
+                y = F.linear(v.transpose(0, 1).reshape(T, m.heads * m.vdim),
+                             L.out_w)
+            else:
+                zxg = F.linear(hm, L.in_w)
+                a = SM.mingru_scan(zxg, L.in_b, self.slots.recurrent[i], cu,
+                                   slots, dt)
+                y = F.linear(a, L.out_w)
+            f = None
+            if ls.mlp is not None:
+                idx, wts = SM.moe_route(hb, L.router_w, L.router_b, ls.mlp.top)
+                f = SM.moe_experts(hb, idx, wts, L.exp_gu, L.exp_down)
+            if i < last:
+                h32, hb = SM.gated_residual_norm(
+                    x, y, f, gates, L.gate_b, mult, M.layers[i + 1].norm_w,
+                    eps, dt)
+            else:
+                SM.gated_residual_add(x, y, f, gates, L.gate_b, mult)
+            if capture is not None:
+                capture.append(x.clone())
+        if want_rows.numel() == 0:
+            return torch.empty(0, S.vocab_size, dtype=torch.float32,
+                               device=x.device)
+        _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, eps, dt)
+        return F.linear(hb, M.head).float()
+
+    # ----------------------------------------------------------- generate
+
+    @torch.no_grad()
+    def generate(self, prompts: List[List[int]], sp: SamplingParams,
+                 eos_token_id: Optional[int] = None,
+                 prefill_token_budget: Optional[int] = None,
+                 stream_cb=None,
+                 token_limits: Optional[List[List[int]]] = None,
+                 cancel_check=None) -> List[List[List[int]]]:
+        """Generate ``sp.n`` completions per prompt (same contract as the
+        dense ``Engine.generate``: candidate order, EOS included when
+        emitted, ``stream_cb(prompt, cand, new_ids)``, per-candidate
+        ``token_limits``, ``cancel_check(prompt)`` polled every step)."""
+        try:
+            return self._generate_inner(prompts, sp, eos_token_id,
+                                        prefill_token_budget, stream_cb,
+                                        token_limits, cancel_check)
+        except Exception:
+            self.reset()   # a failed call strands its sequences; calls are serialized
+            raise
+
+    def _generate_inner(self, prompts, sp, eos, budget, stream_cb,
+                        token_limits, cancel_check):
+        if token_limits is not None:
+            if len(token_limits) != len(prompts):
+                raise ValueError("token_limits must have one list per prompt")
+            for per in token_limits:
+                if len(per) != sp.n or any(
+                        not (1 <= int(v) <= sp.max_tokens) for v in per):
+                    raise ValueError("each token_limits entry needs sp.n caps "
+                                     f"in [1, {sp.max_tokens}]")
+        if sp.n > self.slots.num_slots:
+            raise ValueError(f"SamplingParams.n={sp.n} exceeds the engine's "
+                             f"{self.slots.num_slots} state slots")
+        if any(len(p) == 0 for p in prompts):
+            raise ValueError("empty prompt")
+        if sp.seed is not None:
+            self.generator.manual_seed(int(sp.seed))
+        budget = int(budget or self.cfg.step_token_budget)
+        bs = self.pool.block_size
+        max_total = self.cfg.max_seq_length
+        blocks_for = LatentCachePool.blocks_for
+        results = [[None] * sp.n for _ in prompts]
+        waiting = list(range(len(prompts)))
+        prefilling: List[Sequence] = []    # prompt not fully run yet
+        running: List[Sequence] = []       # decoding candidates
+
+        def worst_blocks(q):
+            return blocks_for(min(len(q.prompt_ids) + sp.max_tokens, max_total), bs)
+
+        def reserved_blocks():
+            need = 0
+            for q in running + prefilling:
+                need += worst_blocks(q) - len(q.block_table)
+            for q in prefilling:
+                need += (sp.n - 1) * (worst_blocks(q) - len(q.prompt_ids) // bs)
+            return need
+
+        def admit():
+            if cancel_check is not None:
+                for pi in [p for p in waiting if cancel_check(p)]:
+                    waiting.remove(pi)
+                    results[pi] = [[] for _ in range(sp.n)]
+            while waiting:
+                pi = waiting[0]
+                L = min(len(prompts[pi]), max_total - 1)
+                worst = blocks_for(min(L + sp.max_tokens, max_total), bs)
+                need = worst + (sp.n - 1) * (worst - L // bs)
+                free_slots = self.slots.num_free - (sp.n - 1) * len(prefilling)
+                if (need > self.pool.allocator.num_free - reserved_blocks()
+                        or free_slots < sp.n):
+                    break
+                waiting.pop(0)
+                prefilling.append(self.open_sequence(prompts[pi][:L], pi))
+
+        def retire(q):
+            results[q.parent_prompt][q.cand_index] = q.output_ids
+            self.close_sequence(q)
+
+        def accept(q, tok):
+            """Append a sampled token; True if the candidate goes on."""
+            q.output_ids.append(tok)
+            if stream_cb is not None:
+                stream_cb(q.parent_prompt, q.cand_index, [tok])
+            done = ((eos is not None and tok == eos)
+                    or len(q.output_ids) >= (q.max_tokens or sp.max_tokens)
+                    or q.total_len >= max_total)
+            if done:
+                retire(q)
+            return not done
+
+        while waiting or prefilling or running:
+            if cancel_check is not None:
+                for q in [q for q in running if cancel_check(q.parent_prompt)]:
+                    running.remove(q)
+                    retire(q)
+                for q in [q for q in prefilling if cancel_check(q.parent_prompt)]:
+                    prefilling.remove(q)
+                    results[q.parent_prompt] = [[] for _ in range(sp.n)]
+                    self.close_sequence(q)
+            admit()
+            work, want, kinds = [], [], []
+            left = budget
+            for q in running:
+                work.append((q, [q.output_ids[-1]]))
+                want.append([0])
+                kinds.append("decode")
+                left -= 1
+            for q in prefilling:
+                if left <= 0 and work:
+                    break
+                rest = len(q.prompt_ids) - q.context_len
+                n = min(rest, max(left, 1))
+                work.append((q, q.prompt_ids[q.context_len:q.context_len + n]))
+                want.append([n - 1] if n == rest else [])
+                kinds.append("last" if n == rest else "part")
+                left -= n
+            if not work:
+                if waiting:
+                    raise MemoryError("cache or slot pool too small to admit "
+                                      "any waiting prompt")
+                break
+            with trace_range(f"hybrid/step[{len(work)}]"):
+                logits = self.step(work, want)
+            # one sampler call: a finished prompt's row is drawn n times
+            src, row = [], 0
+            for k in kinds:
+                if k != "part":
+                    src += [row] * (sp.n if k == "last" else 1)
+                    row += 1
+            toks = OF.sample_tokens(
+                logits[torch.tensor(src, dtype=torch.long, device=logits.device)]
+                .contiguous(), sp.temperature, sp.top_p, sp.top_k,
+                generator=self.generator).tolist() if src else []
+            at = 0
+            still = []
+            for (q, _), kind in zip(work, kinds):
+                if kind == "part":
+                    continue
+                if kind == "decode":
+                    if accept(q, toks[at]):
+                        still.append(q)
+                    at += 1
+                    continue
+                prefilling.remove(q)
+                cands = [q] + [self.fork_sequence(q) for _ in range(sp.n - 1)]
+                for ci, c in enumerate(cands):
+                    c.cand_index = ci
+                    if token_limits is not None:
+                        c.max_tokens = int(token_limits[q.parent_prompt][ci])
+                    if accept(c, toks[at + ci]):
+                        still.append(c)
+                at += sp.n
+            running = still
+        return results

@@ -96,7 +96,7 @@ class Sequence:
 
     __slots__ = ("seq_id", "prompt_ids", "output_ids", "block_table",
                  "context_len", "finished", "parent_prompt",
-                 "last_logits_idx", "cand_index", "max_tokens")
+                 "last_logits_idx", "cand_index", "max_tokens", "slot")
 
     def __init__(self, seq_id: int, prompt_ids: List[int], parent_prompt: int):
         self.seq_id = seq_id
@@ -109,6 +109,7 @@ class Sequence:
         self.last_logits_idx: Optional[int] = None
         self.cand_index = 0  # which of the n candidates of its prompt
         self.max_tokens: Optional[int] = None  # per-seq cap (None -> sp)
+        self.slot: Optional[int] = None  # recurrent-state slot (hybrid models)
 
     @property
     def total_len(self) -> int:

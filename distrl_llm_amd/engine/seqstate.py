@@ -1,0 +1,102 @@
+"""Per-sequence state of layer-list models: latent pages + state slots.
+
+Two pools, both handed out and taken back by the engine as sequences
+come and go:
+
+* :class:`LatentCachePool` — paged rows ``[latent | rotated key part]``
+  for every attention layer that owns a cache (layers that read another
+  layer's cache own none). Block ids come from the same refcounting
+  :class:`BlockAllocator` as the dense models' K/V pool, so a forked
+  candidate shares its prompt's full pages.
+* :class:`StateSlotPool` — fixed-size fp32 state per live sequence: the
+  last ``taps - 1`` inputs of every layer's short convolution and the
+  state vector of every recurrent layer. A slot is zeroed when it is
+  handed out, so whatever its previous owner left cannot leak.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from ..models.hybrid import HybridSpec, LatentAttentionSpec, MinGRUSpec
+from .kvcache import BlockAllocator
+
+
+class LatentCachePool:
+    def __init__(self, spec: HybridSpec, num_blocks: int, block_size: int,
+                 dtype: torch.dtype, device):
+        self.num_blocks = num_blocks
+        self.block_size = block_size
+        self.allocator = BlockAllocator(num_blocks)
+        # layer index -> [num_blocks * block_size, kv_rank + rot_dim]
+        self.rows: Dict[int, torch.Tensor] = {}
+        for i, ls in enumerate(spec.layers):
+            m = ls.mixer
+            if isinstance(m, LatentAttentionSpec) and m.kv_from is None:
+                self.rows[i] = torch.zeros(num_blocks * block_size, m.cache_width,
+                                           dtype=dtype, device=device)
+
+    def layer_rows(self, spec: HybridSpec, layer: int) -> torch.Tensor:
+        m = spec.layers[layer].mixer
+        return self.rows[layer if m.kv_from is None else m.kv_from]
+
+    @staticmethod
+    def blocks_for(num_tokens: int, block_size: int) -> int:
+        return (num_tokens + block_size - 1) // block_size
+
+    @staticmethod
+    def bytes_per_block(spec: HybridSpec, block_size: int, dtype) -> int:
+        w = sum(ls.mixer.cache_width for ls in spec.layers
+                if isinstance(ls.mixer, LatentAttentionSpec)
+                and ls.mixer.kv_from is None)
+        return max(1, w) * block_size * torch.tensor([], dtype=dtype).element_size()
+
+    def copy_block(self, src: int, dst: int) -> None:
+        bs = self.block_size
+        for t in self.rows.values():
+            t[dst * bs:(dst + 1) * bs].copy_(t[src * bs:(src + 1) * bs])
+
+
+class StateSlotPool:
+    def __init__(self, spec: HybridSpec, num_slots: int, device):
+        self.num_slots = num_slots
+        D, k = spec.width, spec.conv_taps - 1
+        # conv tails: one tensor per layer, [slots, taps-1, width] fp32
+        self.tails: List[torch.Tensor] = [
+            torch.zeros(num_slots, k, D, dtype=torch.float32, device=device)
+            for _ in spec.layers]
+        # recurrent state: layer index -> [slots, width] fp32
+        self.recurrent: Dict[int, torch.Tensor] = {
+            i: torch.zeros(num_slots, ls.mixer.width, dtype=torch.float32,
+                           device=device)
+            for i, ls in enumerate(spec.layers)
+            if isinstance(ls.mixer, MinGRUSpec)}
+        self._free = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def _tensors(self):
+        return list(self.tails) + list(self.recurrent.values())
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise MemoryError("state slot pool exhausted")
+        s = self._free.pop()
+        for t in self._tensors():
+            t[s].zero_()
+        return s
+
+    def free(self, slot: int) -> None:
+        assert slot not in self._free
+        self._free.append(slot)
+
+    def copy(self, src: int, dst: int) -> None:
+        for t in self._tensors():
+            t[dst].copy_(t[src])
+
+    def reset(self) -> None:
+        self._free = list(range(self.num_slots - 1, -1, -1))

@@ -1,0 +1,356 @@
+"""Layer-list ("hybrid") decoder models: every layer names its own mixer.
+
+The dense families in ``model.py`` repeat one block; the models here are
+described by a list of layers, each with a token mixer of some kind
+(windowed latent attention, a minGRU recurrence, ...) and an optional
+mixture-of-experts feed-forward. A design is a small table that maps its
+``config.json`` onto these generic layer specs and its tensor names onto
+the packed weights the engine's step function reads; the mechanisms
+themselves (``ops/seqmix.py``) take every size and constant as a
+parameter, so another design can reuse them in another order.
+
+``Nibalix`` is the first design of this kind:
+
+* residual stream in fp32; one offset-weight RMS norm per layer feeds both
+  sublayers (parallel arrangement), ``x += m * (g1*mixer + g2*ff)`` with
+  sigmoid gates read from the normed input;
+* the mixer reads ``h + conv(h)``, a short causal depthwise convolution;
+* mixers: latent attention (a low-rank latent plus one rotated key part
+  shared by the heads is all that is cached; sliding window; a layer may
+  read another layer's cache) and minGRU (gates depend on the current
+  token only; fp32 state carried per sequence);
+* feed-forward: top-k mixture of SiLU-gated experts, softmax over the
+  chosen logits.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn as nn
+
+
+# ------------------------------------------------------------------ specs
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    heads: int
+    dim: int            # unrotated q/k dims per head
+    rot_dim: int        # rotated q/k dims per head (the key part is shared)
+    vdim: int
+    kv_rank: int
+    scale: float
+    rope_base: float
+    rope_dims: int      # how many of the rot_dim entries are rotated
+    window: int         # 0 = unbounded causal
+    kv_from: Optional[int] = None   # layer whose cache this layer reads
+
+    kind = "latent_attention"
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * (self.dim + self.rot_dim)
+
+    @property
+    def cache_width(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass(frozen=True)
+class MinGRUSpec:
+    width: int
+    kind = "mingru"
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    experts: int
+    top: int
+    ff: int
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    mixer: object
+    mlp: Optional[MoESpec]
+
+
+@dataclass(frozen=True)
+class HybridSpec:
+    name: str
+    vocab_size: int
+    width: int
+    norm_eps: float
+    residual_mult: float
+    conv_taps: int
+    layers: tuple = field(default_factory=tuple)
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+
+def nibalix_spec_from_config(cfg: dict, name: str = "nibalix") -> HybridSpec:
+    """Map a Nibalix ``config.json`` onto the generic layer specs."""
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc = lc["mixer"]
+        if lc["type"] == "latent_attention":
+            rot = mc.get("rot") or {}
+            mixer = LatentAttentionSpec(
+                heads=int(mc["heads"]), dim=int(mc["dim"]),
+                rot_dim=int(mc["rot_dim"]), vdim=int(mc["vdim"]),
+                kv_rank=int(mc["kv_rank"]), scale=float(mc["scale"]),
+                rope_base=float(rot.get("base", 10000.0)),
+                rope_dims=int(rot.get("dims", mc["rot_dim"])),
+                window=int((mc.get("mask") or {}).get("size", 0)),
+                kv_from=(int(mc["kv_from"]) if mc.get("kv_from") is not None
+                         else None))
+            if mixer.rope_dims > mixer.rot_dim or mixer.rope_dims % 2:
+                raise ValueError(f"layer {i}: rot.dims must be even and "
+                                 f"<= rot_dim")
+        elif lc["type"] == "mingru":
+            mixer = MinGRUSpec(width=int(mc["width"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {lc['type']!r}")
+        fc = lc.get("mlp")
+        mlp = None
+        if fc is not None:
+            if fc.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: unknown mlp kind {fc['kind']!r}")
+            mlp = MoESpec(experts=int(fc["router"]["experts"]),
+                          top=int(fc["router"]["top"]),
+                          ff=int(fc["expert"]["ff"]))
+            if not 1 <= mlp.top <= mlp.experts:
+                raise ValueError(f"layer {i}: top must be in [1, experts]")
+        layers.append(LayerSpec(mixer, mlp))
+    for i, ls in enumerate(layers):
+        m = ls.mixer
+        if isinstance(m, LatentAttentionSpec) and m.kv_from is not None:
+            src = layers[m.kv_from].mixer if 0 <= m.kv_from < i else None
+            if (not isinstance(src, LatentAttentionSpec)
+                    or src.kv_from is not None
+                    or src.cache_width != m.cache_width
+                    or src.kv_rank != m.kv_rank):
+                raise ValueError(f"layer {i}: kv_from must name an earlier "
+                                 f"latent layer with a cache of its own and "
+                                 f"equal kv_rank/rot_dim")
+    return HybridSpec(name=name, vocab_size=int(cfg["vocab"]),
+                      width=int(cfg["width"]),
+                      norm_eps=float(cfg["norm"]["eps"]),
+                      residual_mult=float(cfg["residual_mult"]),
+                      conv_taps=int(cfg["canon"]["taps"]),
+                      layers=tuple(layers))
+
+
+def nibalix_config_from_spec(spec: HybridSpec) -> dict:
+    """Inverse of :func:`nibalix_spec_from_config` (checkpoint saving)."""
+    layers = []
+    for ls in spec.layers:
+        m = ls.mixer
+        if isinstance(m, LatentAttentionSpec):
+            mc = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim,
+                  "vdim": m.vdim, "kv_rank": m.kv_rank, "scale": m.scale,
+                  "rot": {"base": m.rope_base, "dims": m.rope_dims}}
+            if m.window:
+                mc["mask"] = {"size": m.window}
+            if m.kv_from is not None:
+                mc["kv_from"] = m.kv_from
+            typ = "latent_attention"
+        else:
+            mc, typ = {"width": m.width}, "mingru"
+        fc = None
+        if ls.mlp is not None:
+            fc = {"kind": "moe", "expert": {"ff": ls.mlp.ff},
+                  "router": {"experts": ls.mlp.experts, "top": ls.mlp.top}}
+        layers.append({"type": typ, "mixer": mc, "mlp": fc})
+    return {"architecture": "Nibalix", "canon": {"taps": spec.conv_taps},
+            "layers": layers, "norm": {"eps": spec.norm_eps},
+            "residual_mult": spec.residual_mult, "vocab": spec.vocab_size,
+            "width": spec.width}
+
+
+# ---------------------------------------------------------------- weights
+
+class HybridLayer(nn.Module):
+    """Packed inference weights of one layer.
+
+    Projections that read the same input are stacked along the output
+    axis so each input feeds one GEMM: ``gate_w`` = [rg1; rg2] on the
+    normed input, ``in_w`` = [q; dkv] (latent) or [z; x; g] (minGRU) on
+    the convolved input, ``exp_gu`` = per expert [gate; up]."""
+
+    def __init__(self, spec: HybridSpec, ls: LayerSpec, dtype, device):
+        super().__init__()
+        D = spec.width
+
+        def P(*shape, dt=dtype):
+            return nn.Parameter(torch.zeros(*shape, dtype=dt, device=device),
+                                requires_grad=False)
+
+        f32 = torch.float32
+        self.norm_w = P(D, dt=f32)
+        self.conv_w = P(D, spec.conv_taps, dt=f32)
+        n_gate = 2 * D if ls.mlp is not None else D
+        self.gate_w, self.gate_b = P(n_gate, D), P(n_gate, dt=f32)
+        m = ls.mixer
+        if isinstance(m, LatentAttentionSpec):
+            own = m.kv_from is None
+            self.in_w = P(m.q_size + (m.cache_width if own else 0), D)
+            if own:
+                self.latent_norm_w = P(m.kv_rank, dt=f32)
+            self.uk = P(m.heads, m.dim, m.kv_rank)
+            self.uv = P(m.heads, m.vdim, m.kv_rank)
+            self.out_w = P(D, m.heads * m.vdim)
+        else:
+            self.in_w, self.in_b = P(3 * m.width, D), P(3 * m.width, dt=f32)
+            self.out_w = P(D, m.width)
+        if ls.mlp is not None:
+            f = ls.mlp
+            self.router_w, self.router_b = P(f.experts, D, dt=f32), P(f.experts, dt=f32)
+            self.exp_gu = P(f.experts, 2 * f.ff, D)
+            self.exp_down = P(f.experts, D, f.ff)
+
+
+class HybridLM(nn.Module):
+    """Inference weights of a layer-list model. ``dtype`` is the matrix
+    dtype (bf16 or fp32); norm, conv, bias and router tensors stay fp32."""
+
+    def __init__(self, spec: HybridSpec, dtype: torch.dtype = torch.bfloat16,
+                 device=None):
+        super().__init__()
+        self.spec = spec
+        self.dtype_ = dtype
+        D = spec.width
+        f32 = torch.float32
+
+        def P(*shape, dt=dtype):
+            return nn.Parameter(torch.zeros(*shape, dtype=dt, device=device),
+                                requires_grad=False)
+
+        self.embed = P(spec.vocab_size, D)
+        self.embed_norm_w = P(D, dt=f32)
+        self.final_norm_w = P(D, dt=f32)
+        self.head = P(spec.vocab_size, D)
+        self.layers = nn.ModuleList(
+            [HybridLayer(spec, ls, dtype, device) for ls in spec.layers])
+
+    @property
+    def device(self):
+        return self.embed.device
+
+    # ---- the design's tensor names <-> packed weights -------------------
+
+    def _named_slices(self) -> Dict[str, tuple]:
+        """{checkpoint tensor name: (packed parameter, row0, rows | None)}.
+        ``rows`` None means the tensor fills the whole parameter; expert
+        entries carry an index tuple instead of a row range."""
+        out = {"embed": (self.embed, None), "embed.norm": (self.embed_norm_w, None),
+               "final.norm": (self.final_norm_w, None), "head": (self.head, None)}
+        D = self.spec.width
+        for i, (ls, L) in enumerate(zip(self.spec.layers, self.layers)):
+            p = f"l{i}."
+            out[p + "norm1"] = (L.norm_w, None)
+            out[p + "canon1"] = (L.conv_w, None)
+            out[p + "rg1"], out[p + "rg1.b"] = (L.gate_w, (0, D)), (L.gate_b, (0, D))
+            m = ls.mixer
+            if isinstance(m, LatentAttentionSpec):
+                out[p + "mix.q"] = (L.in_w, (0, m.q_size))
+                if m.kv_from is None:
+                    out[p + "mix.dkv"] = (L.in_w, (m.q_size, m.cache_width))
+                    out[p + "mix.dkv.norm"] = (L.latent_norm_w, None)
+                out[p + "mix.uk"] = (L.uk, "flat")
+                out[p + "mix.uv"] = (L.uv, "flat")
+            else:
+                n = m.width
+                for k, nm in enumerate(("z", "x", "g")):
+                    out[p + "mix." + nm] = (L.in_w, (k * n, n))
+                out[p + "mix.z.b"] = (L.in_b, (0, n))
+                out[p + "mix.x.b"] = (L.in_b, (n, n))
+            out[p + "mix.o"] = (L.out_w, None)
+            if ls.mlp is not None:
+                f = ls.mlp
+                out[p + "rg2"], out[p + "rg2.b"] = (L.gate_w, (D, D)), (L.gate_b, (D, D))
+                out[p + "mlp.router"] = (L.router_w, None)
+                out[p + "mlp.router.b"] = (L.router_b, None)
+                for e in range(f.experts):
+                    out[f"{p}mlp.e{e}.gate"] = (L.exp_gu[e], (0, f.ff))
+                    out[f"{p}mlp.e{e}.up"] = (L.exp_gu[e], (f.ff, f.ff))
+                    out[f"{p}mlp.e{e}.down"] = (L.exp_down[e], None)
+        return out
+
+    @staticmethod
+    def _view(param, where):
+        if where is None:
+            return param
+        if where == "flat":
+            return param.view(-1, param.shape[-1])
+        r0, n = where
+        return param[r0:r0 + n]
+
+    @torch.no_grad()
+    def load_tensors(self, tensors: Dict[str, torch.Tensor], strict=True) -> int:
+        names = self._named_slices()
+        for k, v in tensors.items():
+            if k not in names:
+                if strict:
+                    raise ValueError(f"unexpected checkpoint tensor {k!r}")
+                continue
+            dst = self._view(*names[k])
+            if tuple(dst.shape) != tuple(v.shape):
+                raise ValueError(f"shape mismatch for {k}: checkpoint "
+                                 f"{tuple(v.shape)} vs model {tuple(dst.shape)}")
+            dst.copy_(v.to(dst.dtype))
+        missing = set(names) - set(tensors)
+        if strict and missing:
+            raise ValueError(f"checkpoint misses tensors: {sorted(missing)[:8]}")
+        return len(names) - len(missing)
+
+    def export_tensors(self, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+        return {k: self._view(*w).detach().to(dtype).contiguous().cpu()
+                for k, w in self._named_slices().items()}
+
+    @torch.no_grad()
+    def random_init(self, seed: int = 3407) -> "HybridLM":
+        """Deterministic random weights (synthetic benches and tests)."""
+        dev = self.device
+        g = torch.Generator(device=dev).manual_seed(seed)
+        for name, (param, where) in sorted(self._named_slices().items()):
+            dst = self._view(param, where)
+            r = torch.randn(dst.shape, generator=g, dtype=torch.float32, device=dev)
+            if name == "embed":
+                pass
+            elif dst.dim() >= 2 and "canon" not in name:
+                r *= 1.0 / math.sqrt(dst.shape[-1])
+            elif name.endswith("dkv.norm"):
+                r = 1.0 + 0.1 * r
+            else:
+                r *= 0.1
+            dst.copy_(r.to(dst.dtype))
+        return self
+
+
+# ------------------------------------------------------------ checkpoints
+
+def load_nibalix_checkpoint(path: str, dtype=torch.bfloat16, device=None) -> HybridLM:
+    from safetensors.torch import load_file
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    name = os.path.basename(os.path.normpath(path)) or "nibalix"
+    model = HybridLM(nibalix_spec_from_config(cfg, name), dtype=dtype, device=device)
+    tensors = load_file(os.path.join(path, "model.safetensors"))
+    model.load_tensors(tensors)
+    return model
+
+
+def save_nibalix_checkpoint(model: HybridLM, path: str) -> None:
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    save_file(model.export_tensors(), os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(nibalix_config_from_spec(model.spec), f, indent=1)

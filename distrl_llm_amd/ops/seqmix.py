@@ -1,0 +1,100 @@
+"""Sequence-mixing ops for layer-list models: dispatch to the gfx950
+kernels of ``csrc_seqmix`` on a GPU, to ``seqmix_reference`` on the CPU.
+
+A GPU tensor requires the compiled extension: a missing build raises, it
+never falls back to eager torch. Matrix products stay with the vendor
+GEMM (``F.linear`` / ``torch.bmm``); everything between them runs here.
+Every op takes its sizes and constants as arguments, so a new design
+combines them freely.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import seqmix_reference as R
+from .build import get_seqmix_extension
+
+
+def _ext(op: str):
+    ext = get_seqmix_extension()
+    if ext is None:
+        raise RuntimeError(
+            f"seqmix op '{op}' called on a GPU tensor but the gfx950 "
+            f"extension is not built/loadable (python -m distrl_llm_amd.ops.build)")
+    return ext
+
+
+def offset_rmsnorm(x, w, eps, out_dtype):
+    if x.is_cuda:
+        return _ext("offset_rmsnorm").offset_rmsnorm(x, w, eps, out_dtype)
+    return R.offset_rmsnorm(x, w, eps, out_dtype)
+
+
+def causal_tap_conv(h, w, tails, cu, slots, out_dtype):
+    if h.is_cuda:
+        return _ext("causal_tap_conv").causal_tap_conv(h, w, tails, cu, slots,
+                                                       out_dtype)
+    return R.causal_tap_conv(h, w, tails, cu, slots, out_dtype)
+
+
+def latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
+                   positions, rope_base, rope_dims, page_slot, cache):
+    if proj.is_cuda:
+        return _ext("latent_prepare").latent_prepare(
+            proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
+            positions, rope_base, rope_dims, page_slot, cache)
+    return R.latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache,
+                            norm_w, eps, positions, rope_base, rope_dims,
+                            page_slot, cache)
+
+
+def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
+                            block_size, cu, tok_seq, positions, window, scale,
+                            out_dtype):
+    if q_lat.is_cuda:
+        return _ext("latent_window_attention").latent_window_attention(
+            q_lat, q_rot, cache, kv_rank, block_tables, block_size, tok_seq,
+            positions, window, scale, out_dtype)
+    return R.latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
+                                     block_size, cu, positions, window, scale,
+                                     out_dtype)
+
+
+def mingru_scan(zxg, bias, state, cu, slots, out_dtype):
+    if zxg.is_cuda:
+        return _ext("mingru_scan").mingru_scan(zxg, bias, state, cu, slots,
+                                               out_dtype)
+    return R.mingru_scan(zxg, bias, state, cu, slots, out_dtype)
+
+
+def moe_route(h, router_w, router_b, top):
+    if h.is_cuda:
+        return _ext("moe_route").moe_route(h, router_w, router_b, top)
+    return R.moe_route(h, router_w, router_b, top)
+
+
+def moe_experts(h, idx, wts, exp_gu, exp_down):
+    if h.is_cuda:
+        return _ext("moe_experts").moe_experts(h, idx, wts, exp_gu, exp_down)
+    return R.moe_experts(h, idx, wts, exp_gu, exp_down)
+
+
+def gated_residual_add(x, mix, ff, gates, gate_b, mult):
+    if x.is_cuda:
+        _ext("gated_residual_add").gated_residual_add(x, mix, ff, gates,
+                                                      gate_b, mult)
+        return x
+    return R.gated_residual_add(x, mix, ff, gates, gate_b, mult)
+
+
+def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
+                        out_dtype):
+    """Fused layer tail: the gated residual update followed by the next
+    layer's offset RMS norm of the new residual. Returns (fp32, out_dtype)
+    normed rows; x is updated in place."""
+    if x.is_cuda:
+        return _ext("gated_residual_norm").gated_residual_norm(
+            x, mix, ff, gates, gate_b, mult, next_w, eps, out_dtype)
+    R.gated_residual_add(x, mix, ff, gates, gate_b, mult)
+    return R.offset_rmsnorm(x, next_w, eps, out_dtype)
