@@ -173,7 +173,7 @@ class HybridEngine:
         last = S.num_layers - 1
         for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
             hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i], cu,
-                                    slots, dt)
+                                    meta["tok_seq"], slots, dt)
             gates = F.linear(hb, L.gate_w)
             m = ls.mixer
             if isinstance(m, LatentAttentionSpec):

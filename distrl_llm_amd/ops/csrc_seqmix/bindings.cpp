@@ -1,0 +1,47 @@
+// Python bindings of the sequence-mixing kernel library (gfx950).
+#include <torch/extension.h>
+#include <vector>
+
+std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
+                                          double eps, bool out_bf16);
+void gated_residual_add(torch::Tensor x, torch::Tensor mix,
+                        c10::optional<torch::Tensor> ff, torch::Tensor gates,
+                        torch::Tensor gate_b, double mult);
+std::vector<torch::Tensor> gated_residual_norm(
+    torch::Tensor x, torch::Tensor mix, c10::optional<torch::Tensor> ff,
+    torch::Tensor gates, torch::Tensor gate_b, double mult, torch::Tensor next_w,
+    double eps, bool out_bf16);
+torch::Tensor causal_tap_conv(torch::Tensor h, torch::Tensor w, torch::Tensor tails,
+                              torch::Tensor cu, torch::Tensor tok_seq,
+                              torch::Tensor slots, bool out_bf16);
+torch::Tensor latent_prepare(torch::Tensor proj, int64_t heads, int64_t dim,
+                             int64_t rot_dim, int64_t kv_rank, bool own_cache,
+                             c10::optional<torch::Tensor> norm_w, double eps,
+                             torch::Tensor positions, double rope_base,
+                             int64_t rope_dims, torch::Tensor page_slot,
+                             torch::Tensor cache);
+torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
+                                      torch::Tensor cache, int64_t kv_rank,
+                                      torch::Tensor block_tables, int64_t block_size,
+                                      torch::Tensor tok_seq, torch::Tensor positions,
+                                      int64_t window, double scale);
+torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
+                          torch::Tensor cu, torch::Tensor slots);
+std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
+                                     torch::Tensor router_b, int64_t top);
+torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                          torch::Tensor exp_gu, torch::Tensor exp_down);
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("offset_rmsnorm", &offset_rmsnorm, "offset-weight RMS norm -> (fp32, dtype)");
+  m.def("gated_residual_add", &gated_residual_add, "gated parallel-residual update");
+  m.def("gated_residual_norm", &gated_residual_norm,
+        "gated residual update fused with the next offset RMS norm");
+  m.def("causal_tap_conv", &causal_tap_conv, "short causal depthwise conv with slot tails");
+  m.def("latent_prepare", &latent_prepare, "latent cache write + query rotation");
+  m.def("latent_window_attention", &latent_window_attention,
+        "windowed paged attention in latent space");
+  m.def("mingru_scan", &mingru_scan, "minGRU scan with per-slot fp32 state");
+  m.def("moe_route", &moe_route, "fp32 top-k router");
+  m.def("moe_experts", &moe_experts, "grouped-GEMM mixture of SiLU-gated experts");
+}

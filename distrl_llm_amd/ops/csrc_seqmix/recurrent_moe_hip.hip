@@ -1,0 +1,344 @@
+#include "hip/hip_runtime.h"
+// minGRU scan over a flat varlen batch (fp32 state per slot), the fp32
+// top-k router, and the mixture-of-experts feed-forward as two grouped
+// GEMMs over expert-sorted rows (bf16: MFMA 16x16x32 tiles; fp32: plain
+// FMA) followed by a fixed-order weighted combine.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include "seqmix_common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16v8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+namespace {
+
+// ------------------------------------------------------------- minGRU
+// One thread per (sequence row, channel); tokens of the row in order.
+// zxg row = [z | x | g] pre-activations, bias still to add.
+template <typename T>
+__global__ __launch_bounds__(256) void mingru_scan_kernel(
+    const T* __restrict__ zxg, const float* __restrict__ bias,
+    float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ slots, int n, T* __restrict__ out) {
+  const int b = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= n) return;
+  const int t0 = cu[b], t1 = cu[b + 1];
+  if (t1 == t0) return;
+  const int64_t slot = slots[b];
+  const float bz = bias[ch], bx = bias[n + ch], bg = bias[2 * n + ch];
+  float S = state[slot * n + ch];
+  for (int t = t0; t < t1; ++t) {
+    const T* row = zxg + (int64_t)t * 3 * n;
+    const float z = sm_sigmoid(to_f(row[ch]) + bz);
+    const float u = to_f(row[n + ch]) + bx;
+    const float cand = (u >= 0.f) ? u + 0.5f : sm_sigmoid(u);
+    S = (1.0f - z) * S + z * cand;
+    const float g = to_f(row[2 * n + ch]) + bg;
+    out[(int64_t)t * n + ch] = from_f<T>(S * (g * sm_sigmoid(g)));
+  }
+  state[slot * n + ch] = S;
+}
+
+// ------------------------------------------------------------- router
+// One wave per token: fp32 logits, top-k by repeated arg-max (ties: the
+// lowest index), softmax over the chosen logits.
+#define SM_MAX_EXPERTS 256
+template <typename T>
+__global__ __launch_bounds__(64) void moe_route_kernel(
+    const T* __restrict__ h, const float* __restrict__ w,
+    const float* __restrict__ bias, int D, int E, int top,
+    int* __restrict__ idx, float* __restrict__ wts) {
+  __shared__ float z[SM_MAX_EXPERTS];
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x;
+  for (int e = 0; e < E; ++e) {
+    float acc = 0.f;
+    for (int d = lane; d < D; d += 64) acc += to_f(h[t * D + d]) * w[(int64_t)e * D + d];
+    acc = sm_wave_sum(acc);
+    if (lane == 0) z[e] = acc + bias[e];
+  }
+  __syncthreads();
+  if (lane == 0) {
+    float vmax = 0.f, sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e)
+        if (z[e] > bv) { bv = z[e]; best = e; }
+      if (best < 0) best = 0;             // all NaN/-inf: keep the write in range
+      if (k == 0) vmax = bv;
+      const float p = expf(bv - vmax);
+      idx[t * top + k] = best;
+      wts[t * top + k] = p;
+      sum += p;
+      z[best] = -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) wts[t * top + k] /= sum;
+  }
+}
+
+// ------------------------------------------------- grouped GEMM, bf16
+// Rows are sorted by expert: expert e owns rows off[e]..off[e+1]. A
+// workgroup (4 waves) computes a 64-row x 64-column tile of one expert;
+// wave w owns columns w*16..w*16+15 for the four 16-row m-tiles.
+// MODE 0: out[i, f] = silu(a_i . Wg[f]) * (a_i . Wu[f]), a_i = A[src[i]],
+//         W[e] = [gate (N rows); up (N rows)] x K;   out bf16 [M, N]
+// MODE 1: out[i, n] = a_i . W[e][n], a_i = A[i];     out fp32 [M, N]
+// MFMA 16x16x32 bf16 fragments: A lane l -> row l&15, k (l>>4)*8..+7;
+// B lane l -> column l&15, same k; D lane l reg r -> row (l>>4)*4+r, col l&15.
+SM_INLINE bf16v8 load8(const bf16_t* p, int valid, bool vec) {
+  bf16v8 v;
+  if (vec && valid >= 8) {
+    v = *reinterpret_cast<const bf16v8*>(p);
+  } else {
+    #pragma unroll
+    for (int j = 0; j < 8; ++j)
+      v[j] = (j < valid) ? (__bf16)__bfloat162float(p[j]) : (__bf16)0.0f;
+  }
+  return v;
+}
+
+#define GG_BM 64
+#define GG_BK 64
+#define GG_LD 72   // padded LDS row (bf16 elements)
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
+    const bf16_t* __restrict__ A, const int* __restrict__ src,
+    const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
+    int K, void* __restrict__ outp) {
+  __shared__ __attribute__((aligned(16))) bf16_t a_lds[GG_BM * GG_LD];
+  // which expert / row range is this tile?
+  int e = -1, row0 = 0, rows = 0, tiles = 0;
+  for (int i = 0; i < E; ++i) {
+    const int cnt = off[i + 1] - off[i];
+    const int nt = SM_CDIV(cnt, GG_BM);
+    if ((int)blockIdx.x < tiles + nt) {
+      e = i;
+      row0 = off[i] + ((int)blockIdx.x - tiles) * GG_BM;
+      rows = min(GG_BM, off[i + 1] - row0);
+      break;
+    }
+    tiles += nt;
+  }
+  if (e < 0) return;                       // uniform over the workgroup
+  const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63;
+  const int lrow = l & 15, lk = l >> 4;
+  const bool vec = (K % 8) == 0;
+  const int n = blockIdx.y * 64 + wave * 16 + lrow;     // this lane's B column
+  const int Nw = (MODE == 0) ? 2 * N : N;
+  const bf16_t* Wg = W + ((int64_t)e * Nw + (n < N ? n : 0)) * K;
+  const bf16_t* Wu = Wg + (int64_t)N * K;
+  f32x4 acc[4], acc2[4];
+  #pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc2[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int k0 = 0; k0 < K; k0 += GG_BK) {
+    __syncthreads();
+    #pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int r = pass * 32 + (tid >> 3), kc = (tid & 7) * 8;
+      bf16v8 v;
+      if (r < rows) {
+        const int64_t arow = (MODE == 0) ? src[row0 + r] : (row0 + r);
+        v = load8(A + arow * K + k0 + kc, K - (k0 + kc), vec);
+      } else {
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (__bf16)0.0f;
+      }
+      *reinterpret_cast<bf16v8*>(a_lds + r * GG_LD + kc) = v;
+    }
+    __syncthreads();
+    #pragma unroll
+    for (int ks = 0; ks < GG_BK / 32; ++ks) {
+      const int kk = k0 + ks * 32 + lk * 8;
+      if (k0 + ks * 32 >= K) break;
+      bf16v8 bg, bu;
+      const int valid = (n < N) ? K - kk : 0;
+      bg = load8(Wg + kk, valid, vec);
+      if (MODE == 0) bu = load8(Wu + kk, valid, vec);
+      #pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        const bf16v8 a = *reinterpret_cast<const bf16v8*>(
+            a_lds + (mt * 16 + lrow) * GG_LD + ks * 32 + lk * 8);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bg, acc[mt], 0, 0, 0);
+        if (MODE == 0)
+          acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bu, acc2[mt], 0, 0, 0);
+      }
+    }
+  }
+  const int col = blockIdx.y * 64 + wave * 16 + lrow;
+  if (col >= N) return;
+  #pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int r = mt * 16 + lk * 4 + rr;
+      if (r < rows) {
+        const int64_t o = (int64_t)(row0 + r) * N + col;
+        if (MODE == 0) {
+          const float g = acc[mt][rr];
+          reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(g * sm_sigmoid(g) * acc2[mt][rr]);
+        } else {
+          reinterpret_cast<float*>(outp)[o] = acc[mt][rr];
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------- grouped GEMM, fp32
+// One thread per output element; the expert of a row by scanning off[].
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
+    const float* __restrict__ A, const int* __restrict__ src,
+    const float* __restrict__ W, const int* __restrict__ off, int E, int M,
+    int N, int K, float* __restrict__ out) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= (int64_t)M * N) return;
+  const int i = id / N, n = id % N;
+  int e = 0;
+  while (e + 1 < E && i >= off[e + 1]) ++e;
+  const int Nw = (MODE == 0) ? 2 * N : N;
+  const float* a = A + (int64_t)((MODE == 0) ? src[i] : i) * K;
+  const float* wg = W + ((int64_t)e * Nw + n) * K;
+  float g = 0.f, u = 0.f;
+  for (int k = 0; k < K; ++k) {
+    g = fmaf(a[k], wg[k], g);
+    if (MODE == 0) u = fmaf(a[k], wg[(int64_t)N * K + k], u);
+  }
+  out[id] = (MODE == 0) ? g * sm_sigmoid(g) * u : g;
+}
+
+// out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order)
+__global__ __launch_bounds__(256) void moe_combine_kernel(
+    const float* __restrict__ y, const int64_t* __restrict__ inv,
+    const float* __restrict__ wts, int top, int D, float* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k)
+      acc += wts[t * top + k] * y[inv[t * top + k] * D + d];
+    out[t * D + d] = acc;
+  }
+}
+
+}  // namespace
+
+torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
+                          torch::Tensor cu, torch::Tensor slots) {
+  SM_CHECK_CUDA(zxg); SM_CHECK_CUDA(bias); SM_CHECK_F32(bias);
+  SM_CHECK_CUDA(state); SM_CHECK_F32(state);
+  SM_CHECK_CUDA(cu); SM_CHECK_I32(cu); SM_CHECK_CUDA(slots); SM_CHECK_I32(slots);
+  const int64_t T = zxg.size(0);
+  const int n = zxg.size(1) / 3;
+  const int B = slots.numel();
+  TORCH_CHECK(zxg.size(1) == 3 * n && bias.numel() == 3 * n, "mingru_scan: widths");
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == n && cu.numel() == B + 1, "mingru_scan: state/batch layout");
+  auto out = torch::empty({T, n}, zxg.options());
+  if (T == 0 || B == 0) return out;
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  dim3 grid(B, SM_CDIV(n, 256));
+  if (zxg.scalar_type() == at::kBFloat16)
+   hipLaunchKernelGGL(( mingru_scan_kernel<bf16_t>), dim3(grid), dim3(256), 0, stream, 
+        reinterpret_cast<const bf16_t*>(zxg.data_ptr()), bias.data_ptr<float>(),
+        state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), n,
+        reinterpret_cast<bf16_t*>(out.data_ptr()));
+  else {
+    SM_CHECK_F32(zxg);
+   hipLaunchKernelGGL(( mingru_scan_kernel<float>), dim3(grid), dim3(256), 0, stream, 
+        zxg.data_ptr<float>(), bias.data_ptr<float>(), state.data_ptr<float>(),
+        cu.data_ptr<int>(), slots.data_ptr<int>(), n, out.data_ptr<float>());
+  }
+  SM_CHECK_LAUNCH();
+  return out;
+}
+
+std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
+                                     torch::Tensor router_b, int64_t top) {
+  SM_CHECK_CUDA(h); SM_CHECK_CUDA(router_w); SM_CHECK_F32(router_w);
+  SM_CHECK_CUDA(router_b); SM_CHECK_F32(router_b);
+  const int64_t T = h.size(0);
+  const int D = h.size(1);
+  const int E = router_w.size(0);
+  TORCH_CHECK(router_w.size(1) == D && router_b.numel() == E, "moe_route: shapes");
+  TORCH_CHECK(E <= SM_MAX_EXPERTS && top >= 1 && top <= E, "moe_route: experts/top");
+  auto idx = torch::empty({T, top}, h.options().dtype(at::kInt));
+  auto wts = torch::empty({T, top}, h.options().dtype(at::kFloat));
+  if (T == 0) return {idx, wts};
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  if (h.scalar_type() == at::kBFloat16)
+   hipLaunchKernelGGL(( moe_route_kernel<bf16_t>), dim3(T), dim3(64), 0, stream, 
+        reinterpret_cast<const bf16_t*>(h.data_ptr()), router_w.data_ptr<float>(),
+        router_b.data_ptr<float>(), D, E, (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
+  else {
+    SM_CHECK_F32(h);
+   hipLaunchKernelGGL(( moe_route_kernel<float>), dim3(T), dim3(64), 0, stream, 
+        h.data_ptr<float>(), router_w.data_ptr<float>(), router_b.data_ptr<float>(), D, E,
+        (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
+  }
+  SM_CHECK_LAUNCH();
+  return {idx, wts};
+}
+
+torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                          torch::Tensor exp_gu, torch::Tensor exp_down) {
+  SM_CHECK_CUDA(h); SM_CHECK_CUDA(idx); SM_CHECK_I32(idx); SM_CHECK_CUDA(wts); SM_CHECK_F32(wts);
+  SM_CHECK_CUDA(exp_gu); SM_CHECK_CUDA(exp_down);
+  const int64_t T = h.size(0);
+  const int D = h.size(1);
+  const int top = idx.size(1);
+  const int E = exp_gu.size(0);
+  const int ff = exp_gu.size(1) / 2;
+  TORCH_CHECK(exp_gu.dim() == 3 && exp_gu.size(1) == 2 * ff && exp_gu.size(2) == D, "moe_experts: gate/up shape");
+  TORCH_CHECK(exp_down.dim() == 3 && exp_down.size(0) == E && exp_down.size(1) == D &&
+              exp_down.size(2) == ff, "moe_experts: down shape");
+  TORCH_CHECK(idx.size(0) == T && wts.size(0) == T && wts.size(1) == top, "moe_experts: routing shape");
+  TORCH_CHECK(exp_gu.scalar_type() == h.scalar_type() && exp_down.scalar_type() == h.scalar_type(),
+              "moe_experts: dtypes");
+  auto out = torch::empty({T, D}, h.options().dtype(at::kFloat));
+  if (T == 0) return out;
+  const int64_t M = T * top;
+  // sort the (token, choice) pairs by expert; all on the device, no host sync
+  auto flat = idx.reshape({M}).to(at::kLong);
+  auto sorted = flat.sort(/*stable=*/true, /*dim=*/0, /*descending=*/false);
+  auto order = std::get<1>(sorted);                       // sorted row -> pair
+  auto bounds = torch::arange(E + 1, flat.options());
+  auto off = torch::searchsorted(std::get<0>(sorted), bounds).to(at::kInt).contiguous();
+  auto src = order.floor_divide(top).to(at::kInt).contiguous();   // sorted row -> token
+  auto inv = torch::empty_like(order);
+  inv.index_put_({order}, torch::arange(M, order.options()));     // pair -> sorted row
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  auto y = torch::empty({M, D}, out.options());
+  if (h.scalar_type() == at::kBFloat16) {
+    auto act = torch::empty({M, ff}, h.options());
+    const int row_tiles = SM_CDIV(M, GG_BM) + E;
+   hipLaunchKernelGGL(( moe_gemm_bf16_kernel<0>), dim3(dim3(row_tiles, SM_CDIV(ff, 64))), dim3(256), 0, stream, 
+        reinterpret_cast<const bf16_t*>(h.data_ptr()), src.data_ptr<int>(),
+        reinterpret_cast<const bf16_t*>(exp_gu.data_ptr()), off.data_ptr<int>(), E, ff, D,
+        act.data_ptr());
+    SM_CHECK_LAUNCH();
+   hipLaunchKernelGGL(( moe_gemm_bf16_kernel<1>), dim3(dim3(row_tiles, SM_CDIV(D, 64))), dim3(256), 0, stream, 
+        reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr,
+        reinterpret_cast<const bf16_t*>(exp_down.data_ptr()), off.data_ptr<int>(), E, D, ff,
+        y.data_ptr());
+    SM_CHECK_LAUNCH();
+  } else {
+    SM_CHECK_F32(h);
+    auto act = torch::empty({M, ff}, h.options());
+   hipLaunchKernelGGL(( moe_gemm_f32_kernel<0>), dim3(SM_CDIV(M * ff, 256)), dim3(256), 0, stream, 
+        h.data_ptr<float>(), src.data_ptr<int>(), exp_gu.data_ptr<float>(),
+        off.data_ptr<int>(), E, (int)M, ff, D, act.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+   hipLaunchKernelGGL(( moe_gemm_f32_kernel<1>), dim3(SM_CDIV(M * D, 256)), dim3(256), 0, stream, 
+        act.data_ptr<float>(), nullptr, exp_down.data_ptr<float>(), off.data_ptr<int>(), E,
+        (int)M, D, ff, y.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+  }
+ hipLaunchKernelGGL(( moe_combine_kernel), dim3(T), dim3(256), 0, stream, y.data_ptr<float>(), inv.data_ptr<int64_t>(),
+                                            wts.data_ptr<float>(), top, D, out.data_ptr<float>());
+  SM_CHECK_LAUNCH();
+  return out;
+}

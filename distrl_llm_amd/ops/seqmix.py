@@ -25,16 +25,23 @@ def _ext(op: str):
     return ext
 
 
+def _bf16(dtype) -> bool:
+    if dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"seqmix ops run in bfloat16 or float32, not {dtype}")
+    return dtype == torch.bfloat16
+
+
 def offset_rmsnorm(x, w, eps, out_dtype):
     if x.is_cuda:
-        return _ext("offset_rmsnorm").offset_rmsnorm(x, w, eps, out_dtype)
+        return _ext("offset_rmsnorm").offset_rmsnorm(x.contiguous(), w, eps,
+                                                     _bf16(out_dtype))
     return R.offset_rmsnorm(x, w, eps, out_dtype)
 
 
-def causal_tap_conv(h, w, tails, cu, slots, out_dtype):
+def causal_tap_conv(h, w, tails, cu, tok_seq, slots, out_dtype):
     if h.is_cuda:
-        return _ext("causal_tap_conv").causal_tap_conv(h, w, tails, cu, slots,
-                                                       out_dtype)
+        return _ext("causal_tap_conv").causal_tap_conv(
+            h, w, tails, cu, tok_seq, slots, _bf16(out_dtype))
     return R.causal_tap_conv(h, w, tails, cu, slots, out_dtype)
 
 
@@ -54,8 +61,8 @@ def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                             out_dtype):
     if q_lat.is_cuda:
         return _ext("latent_window_attention").latent_window_attention(
-            q_lat, q_rot, cache, kv_rank, block_tables, block_size, tok_seq,
-            positions, window, scale, out_dtype)
+            q_lat.contiguous(), q_rot, cache, kv_rank, block_tables,
+            block_size, tok_seq, positions, window, scale)
     return R.latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                                      block_size, cu, positions, window, scale,
                                      out_dtype)
@@ -63,8 +70,7 @@ def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
 
 def mingru_scan(zxg, bias, state, cu, slots, out_dtype):
     if zxg.is_cuda:
-        return _ext("mingru_scan").mingru_scan(zxg, bias, state, cu, slots,
-                                               out_dtype)
+        return _ext("mingru_scan").mingru_scan(zxg, bias, state, cu, slots)
     return R.mingru_scan(zxg, bias, state, cu, slots, out_dtype)
 
 
@@ -95,6 +101,6 @@ def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
     normed rows; x is updated in place."""
     if x.is_cuda:
         return _ext("gated_residual_norm").gated_residual_norm(
-            x, mix, ff, gates, gate_b, mult, next_w, eps, out_dtype)
+            x, mix, ff, gates, gate_b, mult, next_w, eps, _bf16(out_dtype))
     R.gated_residual_add(x, mix, ff, gates, gate_b, mult)
     return R.offset_rmsnorm(x, next_w, eps, out_dtype)
