@@ -49,6 +49,12 @@ def parse_args():
                         "output-length caps with this mean (e.g. 450 — the "
                         "reference eval's observed mean; 0 = fixed-length "
                         "no-EOS rounds). Measures in-wave retirement.")
+    p.add_argument("--hybrid-bench", type=str, default="",
+                   help="instead of the RL round: prefill/decode tokens/s of "
+                        "the Nibalix design beside the dense model of equal "
+                        "size, at these comma-separated sizes (1k,2k)")
+    p.add_argument("--hybrid-only", type=str, default="",
+                   help="with --hybrid-bench: run only 'nibalix' or 'dense'")
     p.add_argument("--tiny", action="store_true",
                    help="tiny model + short generations (debug only; NOT the "
                         "headline config)")
@@ -57,6 +63,13 @@ def parse_args():
 
 def main():
     args = parse_args()
+    if args.hybrid_bench:
+        from distrl_llm_amd import bench_hybrid
+        dev = torch.device("cuda:0" if torch.cuda.is_available() and not args.cpu
+                           else "cpu")
+        which = (args.hybrid_only,) if args.hybrid_only else ("nibalix", "dense")
+        bench_hybrid.run(args.hybrid_bench.split(","), dev, which=which)
+        return
     rank = int(os.environ.get("RANK", "0"))
     world_size = int(os.environ.get("WORLD_SIZE", str(args.gpus)))
     os.environ.setdefault("MASTER_ADDR", "127.0.0.1")

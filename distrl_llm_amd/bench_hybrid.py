@@ -1,0 +1,120 @@
+"""Prefill and decode throughput of the Nibalix design beside the dense
+transformer of equal size (``bench.py --hybrid-bench``).
+
+Both models get random weights at layer sizes that resemble a real model
+and run through their own engine's ``generate`` — scheduler, cache, step
+function and sampler included. Prefill tokens/s is timed with one output
+token per prompt; decode tokens/s from the extra time of a longer
+generation.
+"""
+
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+from .config import EngineConfig, SamplingParams
+
+# name -> sizes. The dense twin has the same width, depth, head count and
+# head size, and an MLP as wide as the experts one token uses.
+SIZES = {
+    "1k": dict(width=1024, layers=8, heads=8, dim=64, rot_dim=64, vdim=128,
+               kv_rank=256, window=512, experts=8, top=2, ff=512, vocab=32000),
+    "2k": dict(width=2048, layers=8, heads=16, dim=64, rot_dim=64, vdim=128,
+               kv_rank=512, window=1024, experts=8, top=2, ff=1024, vocab=32000),
+}
+
+
+def nibalix_bench_config(s: dict) -> dict:
+    """Layer pattern: latent attention, latent attention, latent attention
+    reading the previous layer's cache, minGRU."""
+    moe = {"kind": "moe", "expert": {"ff": s["ff"]},
+           "router": {"experts": s["experts"], "top": s["top"]}}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 4 == 3:
+            layers.append({"type": "mingru", "mixer": {"width": s["width"]}, "mlp": moe})
+            continue
+        mc = {"heads": s["heads"], "dim": s["dim"], "rot_dim": s["rot_dim"],
+              "vdim": s["vdim"], "kv_rank": s["kv_rank"],
+              "scale": (s["dim"] + s["rot_dim"]) ** -0.5,
+              "rot": {"base": 10000.0, "dims": s["rot_dim"]},
+              "mask": {"size": s["window"]}}
+        if i % 4 == 2:
+            mc["kv_from"] = i - 1
+        layers.append({"type": "latent_attention", "mixer": mc, "mlp": moe})
+    return {"architecture": "Nibalix", "canon": {"taps": 4}, "layers": layers,
+            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": s["vocab"],
+            "width": s["width"]}
+
+
+def _build_hybrid(s, device, max_len, batch):
+    from .engine.hybrid_engine import HybridEngine
+    from .models.hybrid import HybridLM, nibalix_spec_from_config
+    model = HybridLM(nibalix_spec_from_config(nibalix_bench_config(s)),
+                     dtype=torch.bfloat16, device=device).random_init(1)
+    cfg = EngineConfig(max_seq_length=max_len, kv_block_size=16,
+                       num_kv_blocks=batch * ((max_len + 15) // 16) + 8,
+                       num_state_slots=batch, max_num_seqs=batch,
+                       step_token_budget=8192)
+    return HybridEngine(model, cfg, device=device)
+
+
+def _build_dense(s, device, max_len, batch):
+    from .engine.engine import Engine
+    from .models.model import CausalLM
+    from .models.spec import ModelSpec
+    spec = ModelSpec(f"dense-{s['width']}", s["vocab"], s["width"],
+                     s["top"] * s["ff"], s["layers"], s["heads"], s["heads"],
+                     128, 1e4, 1e-5, False, False, max_position=max_len)
+    model = CausalLM(spec, dtype=torch.bfloat16, device=device).random_init(1)
+    cfg = EngineConfig(max_seq_length=max_len, kv_block_size=16,
+                       num_kv_blocks=batch * ((max_len + 15) // 16) + 8,
+                       max_num_seqs=batch)
+    return Engine(model, cfg, device=device)
+
+
+def _timed(engine, prompts, new_tokens, device):
+    sp = SamplingParams(max_tokens=new_tokens, temperature=1.0, n=1)
+    if device.type == "cuda":
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.generate(prompts, sp, eos_token_id=None)
+    if device.type == "cuda":
+        torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def measure(engine, vocab, batch, prompt_len, new_tokens, device):
+    g = torch.Generator().manual_seed(0)
+    prompts = torch.randint(0, vocab, (batch, prompt_len), generator=g).tolist()
+    _timed(engine, prompts[:2], 4, device)                 # warm-up
+    _timed(engine, prompts, new_tokens, device)            # graphs, allocator
+    t_pre = min(_timed(engine, prompts, 1, device) for _ in range(2))
+    t_all = min(_timed(engine, prompts, new_tokens, device) for _ in range(2))
+    dec = max(t_all - t_pre, 1e-9)
+    return {"prefill_tok_s": batch * prompt_len / t_pre,
+            "decode_tok_s": batch * (new_tokens - 1) / dec,
+            "prefill_s": t_pre, "decode_ms_per_step": 1e3 * dec / (new_tokens - 1)}
+
+
+def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("nibalix", "dense")):
+    out = []
+    for name in sizes:
+        s = SIZES[name]
+        max_len = prompt_len + new_tokens + 1
+        for kind in which:
+            eng = (_build_hybrid if kind == "nibalix" else _build_dense)(
+                s, device, max_len, batch)
+            r = measure(eng, s["vocab"], batch, prompt_len, new_tokens, device)
+            line = {"bench": "hybrid", "size": name, "model": kind, "batch": batch,
+                    "prompt_len": prompt_len, "new_tokens": new_tokens, "dtype": "bf16",
+                    "data": "synthetic", **{k: round(v, 3) for k, v in r.items()}}
+            print(json.dumps(line), flush=True)
+            out.append(line)
+            del eng
+            if device.type == "cuda":
+                torch.cuda.empty_cache()
+    return out

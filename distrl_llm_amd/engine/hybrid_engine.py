@@ -151,9 +151,10 @@ class HybridEngine:
         def i32(v):
             return torch.tensor(v, dtype=torch.int32, device=dev)
 
+        tiles, max_tile = SM.query_tiles([len(t) for _, t in work])
         meta = dict(positions=i32(positions), tok_seq=i32(tok_seq),
                     page_slot=i32(page_slot), cu=i32(cu), slots=i32(slot_idx),
-                    block_tables=i32(tables))
+                    block_tables=i32(tables), tiles=i32(tiles), max_tile=max_tile)
         logits = self._forward(torch.tensor(tokens, dtype=torch.long, device=dev),
                                meta, torch.tensor(want_rows, dtype=torch.long,
                                                   device=dev), capture)
@@ -188,7 +189,8 @@ class HybridEngine:
                 q_lat = torch.bmm(q_nope[..., :m.dim].transpose(0, 1), L.uk)
                 o_lat = SM.latent_window_attention(
                     q_lat, q_rot, cache, m.kv_rank, meta["block_tables"], bs,
-                    cu, meta["tok_seq"], pos, m.window, m.scale, dt)
+                    cu, meta["tok_seq"], pos, m.window, m.scale, dt,
+                    tiles=meta["tiles"], max_tile=meta["max_tile"])
                 v = torch.bmm(o_lat, L.uv.transpose(1, 2))
                 y = F.linear(v.transpose(0, 1).reshape(T, m.heads * m.vdim),
                              L.out_w)
@@ -214,6 +216,15 @@ class HybridEngine:
                                device=x.device)
         _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, eps, dt)
         return F.linear(hb, M.head).float()
+
+    def score(self, ids: Seq[int]) -> torch.Tensor:
+        """Teacher-forced logits of every position of one token sequence
+        (fp32 [len, vocab]), run through a temporary sequence."""
+        q = self.open_sequence()
+        try:
+            return self.step([(q, list(ids))], [list(range(len(ids)))])
+        finally:
+            self.close_sequence(q)
 
     # ----------------------------------------------------------- generate
 

@@ -24,7 +24,9 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
                                       torch::Tensor cache, int64_t kv_rank,
                                       torch::Tensor block_tables, int64_t block_size,
                                       torch::Tensor tok_seq, torch::Tensor positions,
-                                      int64_t window, double scale);
+                                      int64_t window, double scale,
+                                      c10::optional<torch::Tensor> tiles,
+                                      int64_t max_tile_queries);
 torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
                           torch::Tensor cu, torch::Tensor slots);
 std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,

@@ -140,6 +140,227 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
   }
 }
 
+
+// ---- tiled kernel (bf16): up to 16 consecutive queries of one sequence and
+// one head per workgroup; NW waves split the key range and are combined at
+// the end. Scores come from MFMA 16x16x32 (bf16 in, fp32 accumulate) on 32
+// keys at a time; the softmax weights stay fp32 and the weighted latent sum
+// is an fp32 FMA loop with the lanes on the latent axis, so every cache row
+// is read once for all queries of the tile.
+// MFMA fragments: A lane l -> row l&15, k (l>>4)*8..+7; B lane l -> column
+// l&15, same k; D lane l reg r -> row (l>>4)*4+r, column l&15.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16v8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+SM_INLINE bf16v8_t lat_load8(const bf16_t* p, int valid, bool vec) {
+  bf16v8_t v;
+  if (vec && valid >= 8) {
+    v = *reinterpret_cast<const bf16v8_t*>(p);
+  } else {
+    #pragma unroll
+    for (int j = 0; j < 8; ++j)
+      v[j] = (j < valid) ? (__bf16)__bfloat162float(p[j]) : (__bf16)0.0f;
+  }
+  return v;
+}
+
+#define LT_TQ 16
+#define LT_KB 32
+template <int RPL>
+__global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
+    const bf16_t* __restrict__ q_lat,   // [H, Tn, r]
+    const float* __restrict__ q_rot,    // [Tn, H, rd]
+    const bf16_t* __restrict__ cache,   // [rows, r + rd]
+    const int* __restrict__ block_tables, int max_nb, int block_size,
+    const int* __restrict__ tiles,      // [ntiles, 3] = (batch row, first token, queries)
+    const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
+    float scale, int nq_cap, bf16_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int W = r + rd;
+  const int Wp = ((W + 31) / 32) * 32 + 8;          // padded query row (bf16)
+  const int NW = blockDim.x >> 6;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const int lrow = l & 15, lk = l >> 4;
+  bf16_t* q_lds = reinterpret_cast<bf16_t*>(smem);                      // [16][Wp]
+  float* wbase = reinterpret_cast<float*>(smem + (size_t)LT_TQ * Wp * 2);
+  float* p_lds = wbase + wave * (LT_TQ * LT_KB + LT_KB + LT_TQ);        // [16][32]
+  int* krow = reinterpret_cast<int*>(p_lds + LT_TQ * LT_KB);            // [32]
+  float* corr_lds = p_lds + LT_TQ * LT_KB + LT_KB;                      // [16]
+  float* comb = wbase + NW * (LT_TQ * LT_KB + LT_KB + LT_TQ);           // combine area
+
+  const int tile = blockIdx.x, hd = blockIdx.y;
+  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
+  const int p0 = positions[t0], plast = p0 + nq - 1;
+  const int lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+  const int nkeys = plast - lo + 1;
+  const int nblk = (nkeys + LT_KB - 1) / LT_KB;
+  const int* bt = block_tables + (int64_t)b * max_nb;
+  const bool vec = (W % 8) == 0;
+
+  // stage the query tile: [latent part | rotated part], zero padded
+  for (int i = threadIdx.x; i < LT_TQ * Wp; i += blockDim.x) {
+    const int q = i / Wp, k = i % Wp;
+    float v = 0.f;
+    if (q < nq) {
+      if (k < r) v = to_f(q_lat[((int64_t)hd * Tn + t0 + q) * r + k]);
+      else if (k < W) v = q_rot[((int64_t)(t0 + q) * H + hd) * rd + (k - r)];
+    }
+    q_lds[i] = __float2bfloat16(v);
+  }
+  __syncthreads();
+
+  float m[4], lsum[4];
+  #pragma unroll
+  for (int rr = 0; rr < 4; ++rr) { m[rr] = -INFINITY; lsum[rr] = 0.f; }
+  float acc[LT_TQ][RPL];
+  #pragma unroll
+  for (int q = 0; q < LT_TQ; ++q)
+    #pragma unroll
+    for (int i = 0; i < RPL; ++i) acc[q][i] = 0.f;
+  const int KS = (W + 31) / 32;
+
+  for (int kb = wave; kb < nblk; kb += NW) {
+    const int j0 = lo + kb * LT_KB;
+    // cache rows of this block's keys (lanes 0..31), clamped to the last key
+    if (l < LT_KB) {
+      const int j = min(j0 + l, plast);
+      krow[l] = bt[j / block_size] * block_size + j % block_size;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes visible to the wave
+    const bf16_t* k0p = cache + (int64_t)krow[lrow] * W;
+    const bf16_t* k1p = cache + (int64_t)krow[16 + lrow] * W;
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < KS; ++ks) {
+      const int f0 = ks * 32 + lk * 8;
+      const bf16v8_t a = *reinterpret_cast<const bf16v8_t*>(q_lds + lrow * Wp + f0);
+      const bf16v8_t b0 = lat_load8(k0p + f0, W - f0, vec);
+      const bf16v8_t b1 = lat_load8(k1p + f0, W - f0, vec);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b0, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, s1, 0, 0, 0);
+    }
+    // mask, online softmax per query row (rows lk*4 + rr; 16 lanes share a row)
+    float pv0[4], pv1[4], cr[4];
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int q = lk * 4 + rr;
+      const int pq = p0 + q;
+      const int ja = j0 + lrow, jb = j0 + 16 + lrow;
+      const bool oka = q < nq && ja <= pq && (window <= 0 || pq - ja < window);
+      const bool okb = q < nq && jb <= pq && (window <= 0 || pq - jb < window);
+      const float sa = oka ? s0[rr] * scale : -INFINITY;
+      const float sb = okb ? s1[rr] * scale : -INFINITY;
+      float bm = fmaxf(sa, sb);
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, SM_WAVE));
+      const float mn = fmaxf(m[rr], bm);
+      const float c = (mn == -INFINITY) ? 1.0f : expf(m[rr] - mn);
+      const float pa = oka ? expf(sa - mn) : 0.f;
+      const float pb = okb ? expf(sb - mn) : 0.f;
+      float ps = pa + pb;
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, SM_WAVE);
+      lsum[rr] = lsum[rr] * c + ps;
+      m[rr] = mn;
+      pv0[rr] = pa; pv1[rr] = pb; cr[rr] = c;
+    }
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int q = lk * 4 + rr;
+      p_lds[q * LT_KB + lrow] = pv0[rr];
+      p_lds[q * LT_KB + 16 + lrow] = pv1[rr];
+      if (lrow == 0) corr_lds[q] = cr[rr];
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    // weighted latent sum: lanes on the latent axis
+    const int nk = min(LT_KB, nkeys - kb * LT_KB);
+    #pragma unroll
+    for (int q = 0; q < LT_TQ; ++q) {
+      if (q < nq) {
+        const float c = corr_lds[q];
+        #pragma unroll
+        for (int i = 0; i < RPL; ++i) acc[q][i] *= c;
+      }
+    }
+    #pragma unroll 2
+    for (int kk = 0; kk < nk; ++kk) {
+      const bf16_t* crow = cache + (int64_t)krow[kk] * W;
+      float cv[RPL];
+      #pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+        const int f = l + 64 * i;
+        cv[i] = (f < r) ? to_f(crow[f]) : 0.f;
+      }
+      #pragma unroll
+      for (int q = 0; q < LT_TQ; ++q) {
+        if (q < nq) {
+          const float pw = p_lds[q * LT_KB + kk];
+          #pragma unroll
+          for (int i = 0; i < RPL; ++i) acc[q][i] = fmaf(pw, cv[i], acc[q][i]);
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // per-row max and sum to LDS (one lane of each 16-lane group writes)
+  float* ml = comb;                                  // [NW][16][2]
+  float* cacc = comb + NW * LT_TQ * 2;               // [NW][nq_cap][r]
+  #pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    if (lrow == 0) {
+      ml[(wave * LT_TQ + lk * 4 + rr) * 2] = m[rr];
+      ml[(wave * LT_TQ + lk * 4 + rr) * 2 + 1] = lsum[rr];
+    }
+  }
+  if (NW > 1) {
+    #pragma unroll
+    for (int q = 0; q < LT_TQ; ++q) {
+      if (q < nq) {
+        #pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+          const int f = l + 64 * i;
+          if (f < r) cacc[((int64_t)wave * nq_cap + q) * r + f] = acc[q][i];
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  #pragma unroll
+  for (int q = 0; q < LT_TQ; ++q) {
+    if (q < nq) {
+      float M = -INFINITY;
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, ml[(w * LT_TQ + q) * 2]);
+      float L = 0.f;
+      for (int w = 0; w < NW; ++w) {
+        const float mw = ml[(w * LT_TQ + q) * 2];
+        if (mw != -INFINITY) L += ml[(w * LT_TQ + q) * 2 + 1] * expf(mw - M);
+      }
+      const float invL = 1.0f / L;
+      #pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+        const int f = l + 64 * i;
+        if (f < r) {
+          float a;
+          if (NW == 1) {
+            a = acc[q][i];
+          } else {
+            a = 0.f;
+            for (int w = 0; w < NW; ++w) {
+              const float mw = ml[(w * LT_TQ + q) * 2];
+              if (mw != -INFINITY)
+                a += cacc[((int64_t)w * nq_cap + q) * r + f] * expf(mw - M);
+            }
+          }
+          out[((int64_t)hd * Tn + t0 + q) * r + f] = __float2bfloat16(a * invL);
+        }
+      }
+    }
+  }
+}
+
 }  // namespace
 
 torch::Tensor latent_prepare(torch::Tensor proj, int64_t heads, int64_t dim,
@@ -189,7 +410,9 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
                                       torch::Tensor cache, int64_t kv_rank,
                                       torch::Tensor block_tables, int64_t block_size,
                                       torch::Tensor tok_seq, torch::Tensor positions,
-                                      int64_t window, double scale) {
+                                      int64_t window, double scale,
+                                      c10::optional<torch::Tensor> tiles,
+                                      int64_t max_tile_queries) {
   SM_CHECK_CUDA(q_lat); SM_CHECK_CUDA(q_rot); SM_CHECK_F32(q_rot); SM_CHECK_CUDA(cache);
   SM_CHECK_CUDA(block_tables); SM_CHECK_I32(block_tables);
   SM_CHECK_CUDA(tok_seq); SM_CHECK_I32(tok_seq); SM_CHECK_CUDA(positions); SM_CHECK_I32(positions);
@@ -207,6 +430,35 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
   if (T == 0) return out;
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
   const size_t lds = (size_t)(r + rd + 64) * sizeof(float) + 64 * sizeof(int);
+  if (q_lat.scalar_type() == at::kBFloat16 && tiles.has_value() && r <= 512) {
+    // tiled MFMA path
+    SM_CHECK_CUDA(*tiles); SM_CHECK_I32(*tiles);
+    TORCH_CHECK(tiles->dim() == 2 && tiles->size(1) == 3, "latent attention: tiles shape");
+    TORCH_CHECK(max_tile_queries >= 1 && max_tile_queries <= LT_TQ, "latent attention: tile size");
+    const int ntiles = tiles->size(0);
+    const int W = r + rd;
+    const int Wp = ((W + 31) / 32) * 32 + 8;
+    // few small tiles (decoding): four waves split each tile's keys
+    const int NW = (max_tile_queries <= 4 && (int64_t)ntiles * H < 4096) ? 4 : 1;
+    const int nq_cap = (int)max_tile_queries;
+    size_t lds2 = (size_t)LT_TQ * Wp * 2 + (size_t)NW * (LT_TQ * LT_KB + LT_KB + LT_TQ) * 4 +
+                  (size_t)NW * LT_TQ * 2 * 4 + (NW > 1 ? (size_t)NW * nq_cap * r * 4 : 0);
+    TORCH_CHECK(lds2 <= 64 * 1024, "latent attention: tile does not fit in LDS");
+    dim3 g2(ntiles, H);
+    #define LT_LAUNCH(RPL)                                                              \
+     hipLaunchKernelGGL(( latent_attention_tiled_kernel<RPL>), dim3(g2), dim3(64 * NW), lds2, stream,                 \
+          reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),   \
+          reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(), \
+          (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),            \
+          positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale, nq_cap, \
+          reinterpret_cast<bf16_t*>(out.data_ptr()))
+    if (r <= 128) LT_LAUNCH(2);
+    else if (r <= 256) LT_LAUNCH(4);
+    else LT_LAUNCH(8);
+    #undef LT_LAUNCH
+    SM_CHECK_LAUNCH();
+    return out;
+  }
   dim3 grid(T, H);
   if (q_lat.scalar_type() == at::kBFloat16)
    hipLaunchKernelGGL(( latent_attention_kernel<bf16_t>), dim3(grid), dim3(64), lds, stream, 

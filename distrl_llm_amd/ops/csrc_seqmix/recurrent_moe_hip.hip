@@ -41,25 +41,34 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
 }
 
 // ------------------------------------------------------------- router
-// One wave per token: fp32 logits, top-k by repeated arg-max (ties: the
-// lowest index), softmax over the chosen logits.
+// One workgroup per token: the waves share the experts' fp32 logits, then
+// one lane picks the top-k by repeated arg-max (ties: the lowest index) and
+// takes the softmax over the chosen logits.
 #define SM_MAX_EXPERTS 256
 template <typename T>
-__global__ __launch_bounds__(64) void moe_route_kernel(
+__global__ __launch_bounds__(256) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ w,
     const float* __restrict__ bias, int D, int E, int top,
     int* __restrict__ idx, float* __restrict__ wts) {
   __shared__ float z[SM_MAX_EXPERTS];
   const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x;
-  for (int e = 0; e < E; ++e) {
-    float acc = 0.f;
-    for (int d = lane; d < D; d += 64) acc += to_f(h[t * D + d]) * w[(int64_t)e * D + d];
-    acc = sm_wave_sum(acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < E; e += 4) {
+    const float* we = w + (int64_t)e * D;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int d = lane;
+    for (; d + 192 < D; d += 256) {
+      a0 = fmaf(to_f(h[t * D + d]), we[d], a0);
+      a1 = fmaf(to_f(h[t * D + d + 64]), we[d + 64], a1);
+      a2 = fmaf(to_f(h[t * D + d + 128]), we[d + 128], a2);
+      a3 = fmaf(to_f(h[t * D + d + 192]), we[d + 192], a3);
+    }
+    for (; d < D; d += 64) a0 = fmaf(to_f(h[t * D + d]), we[d], a0);
+    const float acc = sm_wave_sum((a0 + a1) + (a2 + a3));
     if (lane == 0) z[e] = acc + bias[e];
   }
   __syncthreads();
-  if (lane == 0) {
+  if (threadIdx.x == 0) {
     float vmax = 0.f, sum = 0.f;
     for (int k = 0; k < top; ++k) {
       int best = -1;
@@ -75,6 +84,40 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
       z[best] = -INFINITY;
     }
     for (int k = 0; k < top; ++k) wts[t * top + k] /= sum;
+  }
+}
+
+// Group the (token, choice) pairs by expert in one workgroup: off[e] = first
+// sorted row of expert e, src[row] = token of that row, inv[pair] = its row.
+// The order inside an expert is arbitrary; every row's result is independent
+// of it and the combine reads rows back through inv.
+__global__ __launch_bounds__(1024) void moe_group_kernel(
+    const int* __restrict__ idx, int M, int top, int E, int* __restrict__ off,
+    int* __restrict__ src, int* __restrict__ inv) {
+  __shared__ int cnt[SM_MAX_EXPERTS];
+  __shared__ int start[SM_MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < M; i += blockDim.x)
+    atomicAdd(&cnt[min(max(idx[i], 0), E - 1)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s;
+      off[e] = s;
+      s += cnt[e];
+      cnt[e] = 0;
+    }
+    start[E] = s;
+    off[E] = s;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < M; i += blockDim.x) {
+    const int e = min(max(idx[i], 0), E - 1);
+    const int row = start[e] + atomicAdd(&cnt[e], 1);
+    src[row] = i / top;
+    inv[i] = row;
   }
 }
 
@@ -214,13 +257,13 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
 
 // out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order)
 __global__ __launch_bounds__(256) void moe_combine_kernel(
-    const float* __restrict__ y, const int64_t* __restrict__ inv,
+    const float* __restrict__ y, const int* __restrict__ inv,
     const float* __restrict__ wts, int top, int D, float* __restrict__ out) {
   const int64_t t = blockIdx.x;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k)
-      acc += wts[t * top + k] * y[inv[t * top + k] * D + d];
+      acc += wts[t * top + k] * y[(int64_t)inv[t * top + k] * D + d];
     out[t * D + d] = acc;
   }
 }
@@ -270,12 +313,12 @@ std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
   if (T == 0) return {idx, wts};
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
   if (h.scalar_type() == at::kBFloat16)
-   hipLaunchKernelGGL(( moe_route_kernel<bf16_t>), dim3(T), dim3(64), 0, stream, 
+   hipLaunchKernelGGL(( moe_route_kernel<bf16_t>), dim3(T), dim3(256), 0, stream, 
         reinterpret_cast<const bf16_t*>(h.data_ptr()), router_w.data_ptr<float>(),
         router_b.data_ptr<float>(), D, E, (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
   else {
     SM_CHECK_F32(h);
-   hipLaunchKernelGGL(( moe_route_kernel<float>), dim3(T), dim3(64), 0, stream, 
+   hipLaunchKernelGGL(( moe_route_kernel<float>), dim3(T), dim3(256), 0, stream, 
         h.data_ptr<float>(), router_w.data_ptr<float>(), router_b.data_ptr<float>(), D, E,
         (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
   }
@@ -296,21 +339,22 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
   TORCH_CHECK(exp_down.dim() == 3 && exp_down.size(0) == E && exp_down.size(1) == D &&
               exp_down.size(2) == ff, "moe_experts: down shape");
   TORCH_CHECK(idx.size(0) == T && wts.size(0) == T && wts.size(1) == top, "moe_experts: routing shape");
+  TORCH_CHECK(E <= SM_MAX_EXPERTS, "moe_experts: too many experts");
   TORCH_CHECK(exp_gu.scalar_type() == h.scalar_type() && exp_down.scalar_type() == h.scalar_type(),
               "moe_experts: dtypes");
   auto out = torch::empty({T, D}, h.options().dtype(at::kFloat));
   if (T == 0) return out;
   const int64_t M = T * top;
-  // sort the (token, choice) pairs by expert; all on the device, no host sync
-  auto flat = idx.reshape({M}).to(at::kLong);
-  auto sorted = flat.sort(/*stable=*/true, /*dim=*/0, /*descending=*/false);
-  auto order = std::get<1>(sorted);                       // sorted row -> pair
-  auto bounds = torch::arange(E + 1, flat.options());
-  auto off = torch::searchsorted(std::get<0>(sorted), bounds).to(at::kInt).contiguous();
-  auto src = order.floor_divide(top).to(at::kInt).contiguous();   // sorted row -> token
-  auto inv = torch::empty_like(order);
-  inv.index_put_({order}, torch::arange(M, order.options()));     // pair -> sorted row
+  // group the (token, choice) pairs by expert on the device (no host sync)
+  auto iopt = h.options().dtype(at::kInt);
+  auto off = torch::empty({E + 1}, iopt);
+  auto src = torch::empty({M}, iopt);
+  auto inv = torch::empty({M}, iopt);
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+ hipLaunchKernelGGL(( moe_group_kernel), dim3(1), dim3(1024), 0, stream, idx.data_ptr<int>(), (int)M, top, E,
+                                           off.data_ptr<int>(), src.data_ptr<int>(),
+                                           inv.data_ptr<int>());
+  SM_CHECK_LAUNCH();
   auto y = torch::empty({M, D}, out.options());
   if (h.scalar_type() == at::kBFloat16) {
     auto act = torch::empty({M, ff}, h.options());
@@ -337,7 +381,7 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
         (int)M, D, ff, y.data_ptr<float>());
     SM_CHECK_LAUNCH();
   }
- hipLaunchKernelGGL(( moe_combine_kernel), dim3(T), dim3(256), 0, stream, y.data_ptr<float>(), inv.data_ptr<int64_t>(),
+ hipLaunchKernelGGL(( moe_combine_kernel), dim3(T), dim3(256), 0, stream, y.data_ptr<float>(), inv.data_ptr<int>(),
                                             wts.data_ptr<float>(), top, D, out.data_ptr<float>());
   SM_CHECK_LAUNCH();
   return out;

@@ -56,13 +56,31 @@ def latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
                             page_slot, cache)
 
 
+QUERY_TILE = 16   # most queries of one sequence the tiled kernel takes at once
+
+
+def query_tiles(row_lengths):
+    """Cut each batch row's tokens into tiles of up to QUERY_TILE
+    consecutive queries: [(batch row, first flat token, queries)], and the
+    largest tile."""
+    tiles, at = [], 0
+    for b, n in enumerate(row_lengths):
+        for k in range(0, n, QUERY_TILE):
+            tiles.append((b, at + k, min(QUERY_TILE, n - k)))
+        at += n
+    return tiles, max((t[2] for t in tiles), default=1)
+
+
 def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                             block_size, cu, tok_seq, positions, window, scale,
-                            out_dtype):
+                            out_dtype, tiles=None, max_tile=0):
+    """``tiles`` (int32 [n, 3] from :func:`query_tiles`, with ``max_tile``)
+    selects the tiled MFMA kernel for bf16; without it, or in fp32, the
+    one-wave-per-query kernel runs."""
     if q_lat.is_cuda:
         return _ext("latent_window_attention").latent_window_attention(
             q_lat.contiguous(), q_rot, cache, kv_rank, block_tables,
-            block_size, tok_seq, positions, window, scale)
+            block_size, tok_seq, positions, window, scale, tiles, max_tile)
     return R.latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                                      block_size, cu, positions, window, scale,
                                      out_dtype)

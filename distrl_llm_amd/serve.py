@@ -256,10 +256,14 @@ def create_app(engine, tokenizer, model_name: str,
         if not out_ids:
             return {"tokens": [], "token_logprobs": [],
                     "top_logprobs": [], "text_offset": []}
-        ids = torch.tensor([list(prompt_ids) + list(out_ids)],
-                           device=engine.device)
-        with torch.no_grad():
-            logits = engine.model(ids)[0].float()
+        if hasattr(engine, "score"):
+            # layer-list engines rescore through their own step function
+            logits = engine.score(list(prompt_ids) + list(out_ids))
+        else:
+            ids = torch.tensor([list(prompt_ids) + list(out_ids)],
+                               device=engine.device)
+            with torch.no_grad():
+                logits = engine.model(ids)[0].float()
         lp = torch.log_softmax(logits, -1)
         start = len(prompt_ids) - 1
         tokens, tlp, top = [], [], []
@@ -343,6 +347,23 @@ def main():
 
     device = torch.device("cuda:0" if torch.cuda.is_available() else "cpu")
     dtype = torch.bfloat16 if device.type == "cuda" else torch.float32
+    from .models.registry import hybrid_design_of, load_model_and_engine
+    if hybrid_design_of(args.model) is not None:
+        # a layer-list design: config.json names it, the registry builds
+        # its model and engine (same generate() contract)
+        if args.adapter or args.enable_prefix_caching:
+            raise SystemExit("--adapter / --enable-prefix-caching apply to "
+                             "the dense model families only")
+        model, engine = load_model_and_engine(
+            args.model, EngineConfig(
+                max_seq_length=args.max_seq_length,
+                gpu_memory_utilization=args.gpu_memory_utilization),
+            dtype=dtype, device=device, seed=args.seed)
+        tokenizer = load_tokenizer(args.model, model.spec.vocab_size)
+        import uvicorn
+        uvicorn.run(create_app(engine, tokenizer, args.model),
+                    host=args.host, port=args.port)
+        return
     spec = resolve_spec(args.model)
     lora_r, lora_alpha = 0, 16.0
     if args.adapter:

@@ -221,6 +221,47 @@ def test_attention_matches_oracle_scores(dev):
     assert rel_err(got, want) < tol(dtype)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("r,rd,window,lens", [(128, 32, 100, [300, 1, 37, 2]),
+                                              (104, 24, 45, [70, 16, 17, 1]),
+                                              (320, 64, 0, [50, 3]),
+                                              (72, 20, 33, [1, 1, 1, 1, 1])])
+def test_tiled_attention_kernel_against_plain_op(r, rd, window, lens):
+    """bf16 MFMA tiles (several tiles per row, ragged last tile, four-wave
+    key split for decode-only batches) against the fp32 torch form."""
+    from distrl_llm_amd.ops import seqmix_reference as R
+    H, bs = 3, 16
+    g = torch.Generator().manual_seed(r)
+    ctx = [n + 150 for n in lens]                       # tokens before this step
+    nblk = [(c + bs - 1) // bs for c in ctx]
+    perm = torch.randperm(sum(nblk) + 2, generator=g).tolist()
+    tables, at = [], 0
+    for n in nblk:
+        tables.append(perm[at:at + n] + [0] * (max(nblk) - n))
+        at += n
+    cache = (torch.randn((sum(nblk) + 2) * bs, r + rd, generator=g)).bfloat16()
+    T = sum(lens)
+    q_lat = (torch.randn(H, T, r, generator=g) * 0.3).bfloat16()
+    q_rot = torch.randn(T, H, rd, generator=g) * 0.3
+    pos, ts, cu = [], [], [0]
+    for b, n in enumerate(lens):
+        pos += list(range(ctx[b] - n, ctx[b]))
+        ts += [b] * n
+        cu.append(cu[-1] + n)
+    i32 = lambda v, d: torch.tensor(v, dtype=torch.int32, device=d)
+    want = R.latent_window_attention(q_lat.float(), q_rot, cache.float(), r, i32(tables, "cpu"), bs,
+                                     i32(cu, "cpu"), i32(pos, "cpu"), window, 0.07, torch.float32)
+    tiles, mt = SM.query_tiles(lens)
+    got = SM.latent_window_attention(q_lat.cuda(), q_rot.cuda(), cache.cuda(), r, i32(tables, "cuda"), bs,
+                                     i32(cu, "cuda"), i32(ts, "cuda"), i32(pos, "cuda"), window, 0.07,
+                                     torch.bfloat16, tiles=i32(tiles, "cuda"), max_tile=mt)
+    plain = SM.latent_window_attention(q_lat.cuda(), q_rot.cuda(), cache.cuda(), r, i32(tables, "cuda"), bs,
+                                       i32(cu, "cuda"), i32(ts, "cuda"), i32(pos, "cuda"), window, 0.07,
+                                       torch.bfloat16)
+    assert rel_err(got.float(), want) < 2e-2
+    assert rel_err(plain.float(), want) < 2e-2
+
+
 def test_mingru_scan_portions_and_slots(dev):
     device, dtype = dev
     n, D, T = 7, 16, 12
@@ -251,10 +292,11 @@ def test_mingru_scan_portions_and_slots(dev):
     assert (pre[:, n:2 * n] + bias[n:2 * n] >= 0).any() and (pre[:, n:2 * n] + bias[n:2 * n] < 0).any()
 
 
-@pytest.mark.parametrize("experts,top", [(5, 2), (4, 1), (3, 3), (9, 4)])
-def test_moe(dev, experts, top):
+@pytest.mark.parametrize("experts,top,D,ff", [(5, 2, 16, 10), (4, 1, 16, 10), (3, 3, 16, 10),
+                                              (9, 4, 16, 10), (4, 2, 104, 72), (3, 2, 33, 70)])
+def test_moe(dev, experts, top, D, ff):
     device, dtype = dev
-    D, ff, T = 16, 10, 70
+    T = 70
     cfg = O.make_cfg([O.gru_layer(width=4, experts=experts, top=top, ff=ff)], width=D)
     Wf = O.random_weights(cfg, 7)
     W = {k: v.double() for k, v in Wf.items()}
