@@ -31,6 +31,65 @@ from .kvcache import Sequence
 from .seqstate import LatentCachePool, StateSlotPool
 
 
+class _DecodeGraph:
+    """One captured decode step for a fixed (padded) number of rows.
+
+    All int inputs live in one static device buffer that is refilled by a
+    single copy before each replay; rows beyond the live ones point at the
+    pools' scratch slot and scratch page, so they compute garbage that
+    nothing reads. The state and cache tensors the graph touches are the
+    pools' own storages, which live as long as the engine."""
+
+    def __init__(self, eng: "HybridEngine", rows: int):
+        self.eng, self.rows = eng, rows
+        bs = eng.pool.block_size
+        self.max_nb = eng._max_table_width()
+        flat, self.lay = self._flat([], [], [], [], [])
+        self.host = torch.zeros(len(flat), dtype=torch.int32, pin_memory=True)
+        self.host.copy_(torch.tensor(flat, dtype=torch.int32))
+        self.buf = self.host.to(eng.device)
+        self.copied = torch.cuda.Event()    # the staging buffer's last upload
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):       # lazy initialisation outside the capture
+            self._body()
+            self._body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = self._body()
+
+    def _flat(self, tokens, positions, page_slot, slots, tables):
+        eng, n, pad = self.eng, len(tokens), self.rows - len(tokens)
+        bs = eng.pool.block_size
+        scratch = eng.pool.scratch_block
+        meta = dict(positions=positions + [0] * pad,
+                    tok_seq=list(range(self.rows)),
+                    page_slot=page_slot + [scratch * bs] * pad,
+                    cu=list(range(self.rows + 1)),
+                    slots=slots + [eng.slots.scratch_slot] * pad,
+                    block_tables=tables + [[scratch]] * pad,
+                    tiles=[(b, b, 1) for b in range(self.rows)], max_tile=1)
+        return eng._pack(tokens + [0] * pad, meta, list(range(self.rows)),
+                         max_nb=self.max_nb)
+
+    def _body(self):
+        tok, meta, want = self.eng._views(self.buf, self.lay, 1)
+        return self.eng._forward(tok, meta, want)
+
+    def run(self, tokens, meta):
+        flat, _ = self._flat(tokens, meta["positions"], meta["page_slot"],
+                             meta["slots"], meta["block_tables"])
+        self.copied.synchronize()           # do not overwrite an upload in flight
+        self.host.copy_(torch.tensor(flat, dtype=torch.int32))
+        self.buf.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self.graph.replay()
+        return self.logits[:len(tokens)]
+
+
 class HybridEngine:
     def __init__(self, model: HybridLM, cfg: EngineConfig,
                  device: Optional[torch.device] = None, seed: int = 0):
@@ -50,6 +109,7 @@ class HybridEngine:
         self.pool = LatentCachePool(self.spec, num_blocks, cfg.kv_block_size,
                                     self.dtype, self.device)
         self.slots = StateSlotPool(self.spec, num_slots, self.device)
+        self._decode_graphs = {}     # padded rows -> _DecodeGraph
 
     def _derive_num_blocks(self, num_slots: int) -> int:
         bs = self.cfg.kv_block_size
@@ -106,6 +166,96 @@ class HybridEngine:
         self.pool.allocator.reset()
         self.slots.reset()
 
+    def _max_table_width(self) -> int:
+        """Most pages one sequence can hold: the block-table width of the
+        captured decode steps."""
+        return min(self.pool.num_blocks, LatentCachePool.blocks_for(
+            self.cfg.max_seq_length, self.pool.block_size))
+
+    def _graph_for(self, rows: int) -> _DecodeGraph:
+        padded = 1
+        while padded < min(rows, 8):
+            padded *= 2
+        if rows > 8:
+            padded = (rows + 7) // 8 * 8
+        g = self._decode_graphs.get(padded)
+        if g is None:
+            g = self._decode_graphs[padded] = _DecodeGraph(self, padded)
+        return g
+
+    # ------------------------------------------------------ step planning
+
+    def _plan(self, work, want):
+        """Host-side layout of one step: takes the pages the new tokens
+        need and returns (token ids, int metadata lists, wanted flat rows)."""
+        bs = self.pool.block_size
+        tokens, positions, tok_seq, page_slot, cu = [], [], [], [], [0]
+        slot_idx, want_rows = [], []
+        for b, (q, toks) in enumerate(work):
+            n = len(toks)
+            if n < 1:
+                raise ValueError("every row of a step needs at least one token")
+            p0 = q.context_len
+            need = LatentCachePool.blocks_for(p0 + n, bs)
+            while len(q.block_table) < need:
+                q.block_table.append(self.pool.allocator.alloc())
+            base = cu[-1]
+            if n <= 8:
+                for p in range(p0, p0 + n):
+                    positions.append(p)
+                    page_slot.append(q.block_table[p // bs] * bs + p % bs)
+            else:
+                p = torch.arange(p0, p0 + n, dtype=torch.int64)
+                table = torch.tensor(q.block_table, dtype=torch.int64)
+                positions.extend(p.tolist())
+                page_slot.extend((table[p // bs] * bs + p % bs).tolist())
+            tok_seq.extend([b] * n)
+            tokens.extend(toks)
+            cu.append(base + n)
+            slot_idx.append(q.slot)
+            for w in ([n - 1] if want is None else want[b]):
+                if not 0 <= w < n:
+                    raise ValueError("wanted place outside the row's tokens")
+                want_rows.append(base + w)
+        tiles, max_tile = SM.query_tiles([len(t) for _, t in work])
+        meta = dict(positions=positions, tok_seq=tok_seq, page_slot=page_slot,
+                    cu=cu, slots=slot_idx,
+                    block_tables=[q.block_table for q, _ in work],
+                    tiles=tiles, max_tile=max_tile)
+        return tokens, meta, want_rows
+
+    @staticmethod
+    def _pack(tokens, meta, want_rows, max_nb=None):
+        """All int inputs of a step as one flat list (one host-to-device
+        copy) plus the layout to cut it up again."""
+        if max_nb is None:
+            max_nb = max(len(t) for t in meta["block_tables"])
+        flat, lay = [], {}
+        tables = [v for t in meta["block_tables"]
+                  for v in (t + [0] * (max_nb - len(t)))]
+        tiles = [v for t in meta["tiles"] for v in t]
+        for name, vals in (("tokens", tokens), ("positions", meta["positions"]),
+                           ("tok_seq", meta["tok_seq"]),
+                           ("page_slot", meta["page_slot"]), ("cu", meta["cu"]),
+                           ("slots", meta["slots"]), ("block_tables", tables),
+                           ("tiles", tiles), ("want", want_rows)):
+            lay[name] = (len(flat), len(vals))
+            flat.extend(vals)
+        lay["max_nb"] = max_nb
+        return flat, lay
+
+    @staticmethod
+    def _views(buf, lay, max_tile):
+        def cut(name):
+            a, n = lay[name]
+            return buf[a:a + n]
+        meta = {k: cut(k) for k in ("positions", "tok_seq", "page_slot", "cu",
+                                    "slots")}
+        meta["block_tables"] = cut("block_tables").view(-1, lay["max_nb"])
+        meta["tiles"] = cut("tiles").view(-1, 3)
+        meta["max_tile"] = max_tile
+        return cut("tokens").long(), meta, cut("want").long()
+
     # --------------------------------------------------------------- step
 
     @torch.no_grad()
@@ -119,45 +269,22 @@ class HybridEngine:
         returned (default: the last one). Returns fp32 [sum(want), vocab]
         in row order. ``capture`` (a list) receives the residual stream
         after every layer."""
-        bs = self.pool.block_size
+        tokens, meta, want_rows = self._plan(work, want)
         dev = self.device
-        tokens, positions, tok_seq, page_slot, cu = [], [], [], [], [0]
-        slot_idx, want_rows = [], []
-        for b, (q, toks) in enumerate(work):
-            n = len(toks)
-            if n < 1:
-                raise ValueError("every row of a step needs at least one token")
-            p0 = q.context_len
-            need = LatentCachePool.blocks_for(p0 + n, bs)
-            while len(q.block_table) < need:
-                q.block_table.append(self.pool.allocator.alloc())
-            base = cu[-1]
-            for k in range(n):
-                p = p0 + k
-                positions.append(p)
-                page_slot.append(q.block_table[p // bs] * bs + p % bs)
-            tokens.extend(int(t) for t in toks)
-            tok_seq.extend([b] * n)
-            cu.append(base + n)
-            slot_idx.append(q.slot)
-            for w in ([n - 1] if want is None else want[b]):
-                if not 0 <= w < n:
-                    raise ValueError("wanted place outside the row's tokens")
-                want_rows.append(base + w)
-        max_nb = max(len(q.block_table) for q, _ in work)
-        tables = [q.block_table + [0] * (max_nb - len(q.block_table))
-                  for q, _ in work]
-
-        def i32(v):
-            return torch.tensor(v, dtype=torch.int32, device=dev)
-
-        tiles, max_tile = SM.query_tiles([len(t) for _, t in work])
-        meta = dict(positions=i32(positions), tok_seq=i32(tok_seq),
-                    page_slot=i32(page_slot), cu=i32(cu), slots=i32(slot_idx),
-                    block_tables=i32(tables), tiles=i32(tiles), max_tile=max_tile)
-        logits = self._forward(torch.tensor(tokens, dtype=torch.long, device=dev),
-                               meta, torch.tensor(want_rows, dtype=torch.long,
-                                                  device=dev), capture)
+        if (capture is None and dev.type == "cuda" and not self.cfg.enforce_eager
+                and meta["max_tile"] == 1 and want_rows == list(range(len(work)))
+                and max(len(t) for t in meta["block_tables"])
+                <= self._max_table_width()):
+            # decode-only step: replay the captured step of this batch size
+            # (the graph's output buffer is reused by the next replay)
+            logits = self._graph_for(len(work)).run(tokens, meta).clone()
+            for q, toks in work:
+                q.context_len += len(toks)
+            return logits
+        packed, lay = self._pack(tokens, meta, want_rows)
+        buf = torch.tensor(packed, dtype=torch.int32).to(dev)
+        tok_t, meta_t, want_t = self._views(buf, lay, meta["max_tile"])
+        logits = self._forward(tok_t, meta_t, want_t, capture)
         for q, toks in work:
             q.context_len += len(toks)
         return logits

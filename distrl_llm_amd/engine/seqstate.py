@@ -30,12 +30,15 @@ class LatentCachePool:
         self.num_blocks = num_blocks
         self.block_size = block_size
         self.allocator = BlockAllocator(num_blocks)
-        # layer index -> [num_blocks * block_size, kv_rank + rot_dim]
+        # one page past the allocator's range that no sequence ever owns:
+        # padding rows of a captured decode step write there
+        self.scratch_block = num_blocks
+        # layer index -> [(num_blocks + 1) * block_size, kv_rank + rot_dim]
         self.rows: Dict[int, torch.Tensor] = {}
         for i, ls in enumerate(spec.layers):
             m = ls.mixer
             if isinstance(m, LatentAttentionSpec) and m.kv_from is None:
-                self.rows[i] = torch.zeros(num_blocks * block_size, m.cache_width,
+                self.rows[i] = torch.zeros((num_blocks + 1) * block_size, m.cache_width,
                                            dtype=dtype, device=device)
 
     def layer_rows(self, spec: HybridSpec, layer: int) -> torch.Tensor:
@@ -62,14 +65,15 @@ class LatentCachePool:
 class StateSlotPool:
     def __init__(self, spec: HybridSpec, num_slots: int, device):
         self.num_slots = num_slots
+        self.scratch_slot = num_slots     # never handed out (padding rows)
         D, k = spec.width, spec.conv_taps - 1
-        # conv tails: one tensor per layer, [slots, taps-1, width] fp32
+        # conv tails: one tensor per layer, [slots + 1, taps-1, width] fp32
         self.tails: List[torch.Tensor] = [
-            torch.zeros(num_slots, k, D, dtype=torch.float32, device=device)
+            torch.zeros(num_slots + 1, k, D, dtype=torch.float32, device=device)
             for _ in spec.layers]
-        # recurrent state: layer index -> [slots, width] fp32
+        # recurrent state: layer index -> [slots + 1, width] fp32
         self.recurrent: Dict[int, torch.Tensor] = {
-            i: torch.zeros(num_slots, ls.mixer.width, dtype=torch.float32,
+            i: torch.zeros(num_slots + 1, ls.mixer.width, dtype=torch.float32,
                            device=device)
             for i, ls in enumerate(spec.layers)
             if isinstance(ls.mixer, MinGRUSpec)}

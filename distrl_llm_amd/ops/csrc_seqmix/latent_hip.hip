@@ -166,7 +166,10 @@ SM_INLINE bf16v8_t lat_load8(const bf16_t* p, int valid, bool vec) {
 
 #define LT_TQ 16
 #define LT_KB 32
-template <int RPL>
+// HEADS: the tile's rows are up to 16 heads of ONE token (decoding: the
+// keys of a sequence are read once for all its heads) instead of up to 16
+// consecutive tokens of one head.
+template <int RPL, bool HEADS>
 __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     const bf16_t* __restrict__ q_lat,   // [H, Tn, r]
     const float* __restrict__ q_rot,    // [Tn, H, rd]
@@ -174,7 +177,10 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     const int* __restrict__ block_tables, int max_nb, int block_size,
     const int* __restrict__ tiles,      // [ntiles, 3] = (batch row, first token, queries)
     const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
-    float scale, int nq_cap, bf16_t* __restrict__ out) {
+    float scale, int nq_cap, bf16_t* __restrict__ out,
+    int ksplit, float* __restrict__ part_acc, float* __restrict__ part_ml) {
+  // ksplit > 1 (HEADS only): blockIdx.z takes a contiguous share of the key
+  // blocks and leaves (max, sum, unnormalised latent sum) for the combine
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int W = r + rd;
   const int Wp = ((W + 31) / 32) * 32 + 8;          // padded query row (bf16)
@@ -188,9 +194,11 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
   float* corr_lds = p_lds + LT_TQ * LT_KB + LT_KB;                      // [16]
   float* comb = wbase + NW * (LT_TQ * LT_KB + LT_KB + LT_TQ);           // combine area
 
-  const int tile = blockIdx.x, hd = blockIdx.y;
-  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
-  const int p0 = positions[t0], plast = p0 + nq - 1;
+  const int tile = blockIdx.x;
+  const int hd = HEADS ? blockIdx.y * LT_TQ : blockIdx.y;     // first / only head
+  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1];
+  const int nq = HEADS ? min(LT_TQ, H - hd) : tiles[3 * tile + 2];
+  const int p0 = positions[t0], plast = HEADS ? p0 : p0 + nq - 1;
   const int lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
   const int nkeys = plast - lo + 1;
   const int nblk = (nkeys + LT_KB - 1) / LT_KB;
@@ -202,8 +210,9 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     const int q = i / Wp, k = i % Wp;
     float v = 0.f;
     if (q < nq) {
-      if (k < r) v = to_f(q_lat[((int64_t)hd * Tn + t0 + q) * r + k]);
-      else if (k < W) v = q_rot[((int64_t)(t0 + q) * H + hd) * rd + (k - r)];
+      const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+      if (k < r) v = to_f(q_lat[((int64_t)hq * Tn + tq) * r + k]);
+      else if (k < W) v = q_rot[((int64_t)tq * H + hq) * rd + (k - r)];
     }
     q_lds[i] = __float2bfloat16(v);
   }
@@ -219,7 +228,9 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     for (int i = 0; i < RPL; ++i) acc[q][i] = 0.f;
   const int KS = (W + 31) / 32;
 
-  for (int kb = wave; kb < nblk; kb += NW) {
+  const int kb_lo = (int)(((int64_t)nblk * blockIdx.z) / ksplit);
+  const int kb_hi = (int)(((int64_t)nblk * (blockIdx.z + 1)) / ksplit);
+  for (int kb = kb_lo + wave; kb < kb_hi; kb += NW) {
     const int j0 = lo + kb * LT_KB;
     // cache rows of this block's keys (lanes 0..31), clamped to the last key
     if (l < LT_KB) {
@@ -231,6 +242,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     const bf16_t* k0p = cache + (int64_t)krow[lrow] * W;
     const bf16_t* k1p = cache + (int64_t)krow[16 + lrow] * W;
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    #pragma unroll 4
     for (int ks = 0; ks < KS; ++ks) {
       const int f0 = ks * 32 + lk * 8;
       const bf16v8_t a = *reinterpret_cast<const bf16v8_t*>(q_lds + lrow * Wp + f0);
@@ -244,7 +256,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const int q = lk * 4 + rr;
-      const int pq = p0 + q;
+      const int pq = HEADS ? p0 : p0 + q;
       const int ja = j0 + lrow, jb = j0 + 16 + lrow;
       const bool oka = q < nq && ja <= pq && (window <= 0 || pq - ja < window);
       const bool okb = q < nq && jb <= pq && (window <= 0 || pq - jb < window);
@@ -283,7 +295,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
         for (int i = 0; i < RPL; ++i) acc[q][i] *= c;
       }
     }
-    #pragma unroll 2
+    #pragma unroll 4
     for (int kk = 0; kk < nk; ++kk) {
       const bf16_t* crow = cache + (int64_t)krow[kk] * W;
       float cv[RPL];
@@ -306,7 +318,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
 
   // per-row max and sum to LDS (one lane of each 16-lane group writes)
   float* ml = comb;                                  // [NW][16][2]
-  float* cacc = comb + NW * LT_TQ * 2;               // [NW][nq_cap][r]
+  float* cacc = comb + NW * LT_TQ * 2;               // [NW - 1][nq_cap][r]: waves 1..
   #pragma unroll
   for (int rr = 0; rr < 4; ++rr) {
     if (lrow == 0) {
@@ -314,14 +326,14 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
       ml[(wave * LT_TQ + lk * 4 + rr) * 2 + 1] = lsum[rr];
     }
   }
-  if (NW > 1) {
+  if (wave > 0) {
     #pragma unroll
     for (int q = 0; q < LT_TQ; ++q) {
       if (q < nq) {
         #pragma unroll
         for (int i = 0; i < RPL; ++i) {
           const int f = l + 64 * i;
-          if (f < r) cacc[((int64_t)wave * nq_cap + q) * r + f] = acc[q][i];
+          if (f < r) cacc[((int64_t)(wave - 1) * nq_cap + q) * r + f] = acc[q][i];
         }
       }
     }
@@ -339,25 +351,50 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
         if (mw != -INFINITY) L += ml[(w * LT_TQ + q) * 2 + 1] * expf(mw - M);
       }
       const float invL = 1.0f / L;
+      const int tq_ = HEADS ? t0 : t0 + q, hq_ = HEADS ? hd + q : hd;
+      if (ksplit > 1 && l == 0) {
+        part_ml[(((int64_t)tq_ * H + hq_) * ksplit + blockIdx.z) * 2] = M;
+        part_ml[(((int64_t)tq_ * H + hq_) * ksplit + blockIdx.z) * 2 + 1] = L;
+      }
       #pragma unroll
       for (int i = 0; i < RPL; ++i) {
         const int f = l + 64 * i;
         if (f < r) {
-          float a;
-          if (NW == 1) {
-            a = acc[q][i];
-          } else {
-            a = 0.f;
-            for (int w = 0; w < NW; ++w) {
-              const float mw = ml[(w * LT_TQ + q) * 2];
-              if (mw != -INFINITY)
-                a += cacc[((int64_t)w * nq_cap + q) * r + f] * expf(mw - M);
-            }
+          const float m0 = ml[q * 2];
+          float a = (m0 != -INFINITY) ? acc[q][i] * expf(m0 - M) : 0.f;
+          for (int w = 1; w < NW; ++w) {
+            const float mw = ml[(w * LT_TQ + q) * 2];
+            if (mw != -INFINITY)
+              a += cacc[((int64_t)(w - 1) * nq_cap + q) * r + f] * expf(mw - M);
           }
-          out[((int64_t)hd * Tn + t0 + q) * r + f] = __float2bfloat16(a * invL);
+          if (ksplit > 1)
+            part_acc[(((int64_t)tq_ * H + hq_) * ksplit + blockIdx.z) * r + f] = a;
+          else
+            out[((int64_t)hq_ * Tn + tq_) * r + f] = __float2bfloat16(a * invL);
         }
       }
     }
+  }
+}
+
+// Merge the key splits of one (token, head): out = sum_z acc_z e^(m_z - M) / L.
+__global__ __launch_bounds__(256) void latent_combine_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    int Tn, int H, int r, int ksplit, bf16_t* __restrict__ out) {
+  const int t = blockIdx.x / H, hd = blockIdx.x % H;
+  const float* ml = part_ml + (int64_t)blockIdx.x * ksplit * 2;
+  float M = -INFINITY;
+  for (int z = 0; z < ksplit; ++z) M = fmaxf(M, ml[z * 2]);
+  float L = 0.f;
+  for (int z = 0; z < ksplit; ++z)
+    if (ml[z * 2] != -INFINITY) L += ml[z * 2 + 1] * expf(ml[z * 2] - M);
+  const float invL = 1.0f / L;
+  for (int f = threadIdx.x; f < r; f += blockDim.x) {
+    float a = 0.f;
+    for (int z = 0; z < ksplit; ++z)
+      if (ml[z * 2] != -INFINITY)
+        a += part_acc[((int64_t)blockIdx.x * ksplit + z) * r + f] * expf(ml[z * 2] - M);
+    out[((int64_t)hd * Tn + t) * r + f] = __float2bfloat16(a * invL);
   }
 }
 
@@ -438,24 +475,63 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     const int ntiles = tiles->size(0);
     const int W = r + rd;
     const int Wp = ((W + 31) / 32) * 32 + 8;
-    // few small tiles (decoding): four waves split each tile's keys
-    const int NW = (max_tile_queries <= 4 && (int64_t)ntiles * H < 4096) ? 4 : 1;
-    const int nq_cap = (int)max_tile_queries;
+    // decode-only batches (one query per row): a tile is one token with up
+    // to 16 of its heads, and four waves split its keys
+    const bool heads = max_tile_queries == 1 && H > 1;
+    const int NW = (heads || (max_tile_queries <= 4 && (int64_t)ntiles * H < 4096)) ? 4 : 1;
+    const int nq_cap = heads ? LT_TQ : (int)max_tile_queries;
     size_t lds2 = (size_t)LT_TQ * Wp * 2 + (size_t)NW * (LT_TQ * LT_KB + LT_KB + LT_TQ) * 4 +
-                  (size_t)NW * LT_TQ * 2 * 4 + (NW > 1 ? (size_t)NW * nq_cap * r * 4 : 0);
-    TORCH_CHECK(lds2 <= 64 * 1024, "latent attention: tile does not fit in LDS");
-    dim3 g2(ntiles, H);
-    #define LT_LAUNCH(RPL)                                                              \
-     hipLaunchKernelGGL(( latent_attention_tiled_kernel<RPL>), dim3(g2), dim3(64 * NW), lds2, stream,                 \
+                  (size_t)NW * LT_TQ * 2 * 4 + (size_t)(NW - 1) * nq_cap * r * 4;
+    TORCH_CHECK(lds2 <= 150 * 1024, "latent attention: tile does not fit in LDS");
+    // decode: enough key splits to fill the chip, at most one per wave pass
+    int ksplit = 1;
+    torch::Tensor part_acc, part_ml;
+    float *pacc = nullptr, *pml = nullptr;
+    if (heads) {
+      const int64_t groups = (int64_t)ntiles * SM_CDIV(H, LT_TQ);
+      ksplit = (int)std::min<int64_t>(16, std::max<int64_t>(1, 512 / groups));
+      if (window > 0)
+        ksplit = (int)std::min<int64_t>(ksplit, std::max<int64_t>(1, SM_CDIV(window, LT_KB * NW)));
+      if (ksplit > 1) {
+        part_acc = torch::empty({T, H, ksplit, r}, q_rot.options());
+        part_ml = torch::empty({T, H, ksplit, 2}, q_rot.options());
+        pacc = part_acc.data_ptr<float>();
+        pml = part_ml.data_ptr<float>();
+      }
+    }
+    dim3 g2(ntiles, heads ? SM_CDIV(H, LT_TQ) : H, ksplit);
+    #define LT_LAUNCH(RPL, HD)                                                          \
+      do {                                                                              \
+        auto kern = latent_attention_tiled_kernel<RPL, HD>;                             \
+        static int raised = 0;     /* per kernel variant; not repeated under graph capture */ \
+        if (lds2 > 64 * 1024 && (int)lds2 > raised) {                                   \
+          TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),          \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2) == hipSuccess, \
+                      "latent attention: cannot raise the LDS limit");                  \
+          raised = (int)lds2;                                                           \
+        }                                                                               \
+       hipLaunchKernelGGL(( kern), dim3(g2), dim3(64 * NW), lds2, stream,                                             \
           reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),   \
           reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(), \
           (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),            \
           positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale, nq_cap, \
-          reinterpret_cast<bf16_t*>(out.data_ptr()))
-    if (r <= 128) LT_LAUNCH(2);
-    else if (r <= 256) LT_LAUNCH(4);
-    else LT_LAUNCH(8);
+          reinterpret_cast<bf16_t*>(out.data_ptr()), ksplit, pacc, pml);                \
+      } while (0)
+    if (heads) {
+      if (r <= 128) LT_LAUNCH(2, true);
+      else if (r <= 256) LT_LAUNCH(4, true);
+      else LT_LAUNCH(8, true);
+    } else {
+      if (r <= 128) LT_LAUNCH(2, false);
+      else if (r <= 256) LT_LAUNCH(4, false);
+      else LT_LAUNCH(8, false);
+    }
     #undef LT_LAUNCH
+    if (ksplit > 1) {
+      SM_CHECK_LAUNCH();
+     hipLaunchKernelGGL(( latent_combine_kernel), dim3((int)(T * H)), dim3(256), 0, stream, 
+          pacc, pml, (int)T, H, r, ksplit, reinterpret_cast<bf16_t*>(out.data_ptr()));
+    }
     SM_CHECK_LAUNCH();
     return out;
   }

@@ -55,7 +55,7 @@ def main(argv=None) -> int:
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
     bs = args.block_size
-    cfg = EngineConfig(max_seq_length=1 << 30, kv_block_size=bs,
+    cfg = EngineConfig(max_seq_length=max(args.max_tokens, bs), kv_block_size=bs,
                        num_kv_blocks=max(1, (args.max_tokens + bs - 1) // bs),
                        num_state_slots=args.slots, max_num_seqs=args.slots)
     _model, engine = load_model_and_engine(args.model, cfg, dtype=dtype,

@@ -473,6 +473,35 @@ def test_generate_greedy_through_scheduler(dev):
     assert eng.pool.allocator.num_free == 40 and eng.slots.num_free == 4
 
 
+@pytest.mark.gpu
+def test_captured_decode_equals_eager():
+    """Decode-only steps replay a captured graph; the same schedule run
+    eagerly must give the same logits, replay after replay, also with rows
+    padded onto the scratch slot and page."""
+    cfg = mixed_cfg()
+    dev = ("cuda", torch.float32)
+    W, eng = build(cfg, dev, blocks=40, block_size=4, slots=4)
+    model = eng.model
+    eager = HybridEngine(model, EngineConfig(max_seq_length=4096, kv_block_size=4, num_kv_blocks=40,
+                                             num_state_slots=4, max_num_seqs=4, enforce_eager=True),
+                         device=torch.device("cuda"))
+    prompts = [toks(n, cfg["vocab"], seed=60 + n) for n in (5, 11, 2)]
+    outs = []
+    for e in (eng, eager):
+        qs = [e.open_sequence() for _ in prompts]
+        e.step([(q, p) for q, p in zip(qs, prompts)])
+        got = []
+        for k in range(12):                       # three rows pad to four
+            got.append(e.step([(q, [(7 * k + i) % cfg["vocab"]]) for i, q in enumerate(qs)]))
+            if k == 5:                            # eager work between replays
+                e.step([(qs[0], [1, 2, 3])])
+        for q in qs:
+            e.close_sequence(q)
+        outs.append(torch.stack(got))
+    assert eng._decode_graphs and not eager._decode_graphs
+    assert rel_err(outs[0], outs[1]) < 1e-5
+
+
 def test_checkpoint_registry_and_trace_replay(tmp_path):
     """config.json selects the model class; the replay tool drives the same
     engine from a step trace on standard input."""
