@@ -217,11 +217,14 @@ class HybridEngine:
                 if not 0 <= w < n:
                     raise ValueError("wanted place outside the row's tokens")
                 want_rows.append(base + w)
-        tiles, max_tile = SM.query_tiles([len(t) for _, t in work])
+        lengths = [len(t) for _, t in work]
+        tiles, max_tile = SM.query_tiles(lengths)
+        chunks, chunk_cu = SM.scan_chunks(lengths)
         meta = dict(positions=positions, tok_seq=tok_seq, page_slot=page_slot,
                     cu=cu, slots=slot_idx,
                     block_tables=[q.block_table for q, _ in work],
-                    tiles=tiles, max_tile=max_tile)
+                    tiles=tiles, max_tile=max_tile, scan_chunks=chunks,
+                    scan_cu=chunk_cu)
         return tokens, meta, want_rows
 
     @staticmethod
@@ -238,7 +241,10 @@ class HybridEngine:
                            ("tok_seq", meta["tok_seq"]),
                            ("page_slot", meta["page_slot"]), ("cu", meta["cu"]),
                            ("slots", meta["slots"]), ("block_tables", tables),
-                           ("tiles", tiles), ("want", want_rows)):
+                           ("tiles", tiles), ("want", want_rows),
+                           ("scan_chunks", [v for c in meta.get("scan_chunks", [])
+                                            for v in c]),
+                           ("scan_cu", meta.get("scan_cu", []))):
             lay[name] = (len(flat), len(vals))
             flat.extend(vals)
         lay["max_nb"] = max_nb
@@ -253,6 +259,8 @@ class HybridEngine:
                                     "slots")}
         meta["block_tables"] = cut("block_tables").view(-1, lay["max_nb"])
         meta["tiles"] = cut("tiles").view(-1, 3)
+        meta["scan_chunks"] = cut("scan_chunks").view(-1, 3)
+        meta["scan_cu"] = cut("scan_cu")
         meta["max_tile"] = max_tile
         return cut("tokens").long(), meta, cut("want").long()
 
@@ -324,7 +332,8 @@ class HybridEngine:
             else:
                 zxg = F.linear(hm, L.in_w)
                 a = SM.mingru_scan(zxg, L.in_b, self.slots.recurrent[i], cu,
-                                   slots, dt)
+                                   slots, dt, meta["scan_chunks"],
+                                   meta["scan_cu"])
                 y = F.linear(a, L.out_w)
             f = None
             if ls.mlp is not None:

@@ -28,7 +28,9 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
                                       c10::optional<torch::Tensor> tiles,
                                       int64_t max_tile_queries);
 torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
-                          torch::Tensor cu, torch::Tensor slots);
+                          torch::Tensor cu, torch::Tensor slots,
+                          c10::optional<torch::Tensor> chunks,
+                          c10::optional<torch::Tensor> chunk_cu);
 std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
                                      torch::Tensor router_b, int64_t top);
 torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,

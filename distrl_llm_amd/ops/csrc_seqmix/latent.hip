@@ -165,6 +165,8 @@ SM_INLINE bf16v8_t lat_load8(const bf16_t* p, int valid, bool vec) {
 
 #define LT_TQ 16
 #define LT_KB 32
+// latent entry of accumulator i in lane l: lanes own adjacent pairs
+#define LT_FEAT(l, i) (2 * (l) + 128 * ((i) >> 1) + ((i) & 1))
 // HEADS: the tile's rows are up to 16 heads of ONE token (decoding: the
 // keys of a sequence are read once for all its heads) instead of up to 16
 // consecutive tokens of one head.
@@ -203,17 +205,43 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
   const int nblk = (nkeys + LT_KB - 1) / LT_KB;
   const int* bt = block_tables + (int64_t)b * max_nb;
   const bool vec = (W % 8) == 0;
+  const bool pair = (W % 2) == 0 && (r % 2) == 0;   // 4-byte aligned entry pairs
 
   // stage the query tile: [latent part | rotated part], zero padded
-  for (int i = threadIdx.x; i < LT_TQ * Wp; i += blockDim.x) {
-    const int q = i / Wp, k = i % Wp;
-    float v = 0.f;
-    if (q < nq) {
-      const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
-      if (k < r) v = to_f(q_lat[((int64_t)hq * Tn + tq) * r + k]);
-      else if (k < W) v = q_rot[((int64_t)tq * H + hq) * rd + (k - r)];
+  if ((r % 8) == 0) {
+    // latent part in 16-byte pieces, the rest entry by entry
+    const int r8 = r / 8, w8 = (Wp - r);
+    for (int i = threadIdx.x; i < LT_TQ * r8; i += blockDim.x) {
+      const int q = i / r8, k = (i % r8) * 8;
+      bf16v8_t v;
+      #pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (__bf16)0.0f;
+      if (q < nq) {
+        const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+        v = *reinterpret_cast<const bf16v8_t*>(q_lat + ((int64_t)hq * Tn + tq) * r + k);
+      }
+      *reinterpret_cast<bf16v8_t*>(q_lds + q * Wp + k) = v;
     }
-    q_lds[i] = __float2bfloat16(v);
+    for (int i = threadIdx.x; i < LT_TQ * w8; i += blockDim.x) {
+      const int q = i / w8, k = r + i % w8;
+      float v = 0.f;
+      if (q < nq && k < W) {
+        const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+        v = q_rot[((int64_t)tq * H + hq) * rd + (k - r)];
+      }
+      q_lds[q * Wp + k] = __float2bfloat16(v);
+    }
+  } else {
+    for (int i = threadIdx.x; i < LT_TQ * Wp; i += blockDim.x) {
+      const int q = i / Wp, k = i % Wp;
+      float v = 0.f;
+      if (q < nq) {
+        const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+        if (k < r) v = to_f(q_lat[((int64_t)hq * Tn + tq) * r + k]);
+        else if (k < W) v = q_rot[((int64_t)tq * H + hq) * rd + (k - r)];
+      }
+      q_lds[i] = __float2bfloat16(v);
+    }
   }
   __syncthreads();
 
@@ -294,14 +322,25 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
         for (int i = 0; i < RPL; ++i) acc[q][i] *= c;
       }
     }
-    #pragma unroll 4
+    #pragma unroll 8
     for (int kk = 0; kk < nk; ++kk) {
       const bf16_t* crow = cache + (int64_t)krow[kk] * W;
       float cv[RPL];
-      #pragma unroll
-      for (int i = 0; i < RPL; ++i) {
-        const int f = l + 64 * i;
-        cv[i] = (f < r) ? to_f(crow[f]) : 0.f;
+      if (pair) {                       // two adjacent entries per 4-byte load
+        #pragma unroll
+        for (int i = 0; i < RPL; i += 2) {
+          const int f = LT_FEAT(l, i);
+          uint32_t w2 = 0;
+          if (f < r) w2 = *reinterpret_cast<const uint32_t*>(crow + f);
+          cv[i] = __uint_as_float(w2 << 16);
+          cv[i + 1] = __uint_as_float(w2 & 0xffff0000u);
+        }
+      } else {
+        #pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+          const int f = LT_FEAT(l, i);
+          cv[i] = (f < r) ? to_f(crow[f]) : 0.f;
+        }
       }
       #pragma unroll
       for (int q = 0; q < LT_TQ; ++q) {
@@ -331,7 +370,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
       if (q < nq) {
         #pragma unroll
         for (int i = 0; i < RPL; ++i) {
-          const int f = l + 64 * i;
+          const int f = LT_FEAT(l, i);
           if (f < r) cacc[((int64_t)(wave - 1) * nq_cap + q) * r + f] = acc[q][i];
         }
       }
@@ -357,7 +396,7 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
       }
       #pragma unroll
       for (int i = 0; i < RPL; ++i) {
-        const int f = l + 64 * i;
+        const int f = LT_FEAT(l, i);
         if (f < r) {
           const float m0 = ml[q * 2];
           float a = (m0 != -INFINITY) ? acc[q][i] * expf(m0 - M) : 0.f;

@@ -40,6 +40,79 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
   state[slot * n + ch] = S;
 }
 
+// Chunked form for long rows: a row's tokens are cut into chunks that run
+// in parallel. S_t = a_t S_(t-1) + b_t composes, so a chunk is summarised
+// by (P, Q) with S_end = P S_start + Q (pass 1), the chunk starts follow
+// from a short serial walk over the row's chunks (pass 2), and pass 3
+// redoes each chunk from its true start and writes the outputs.
+template <typename T>
+SM_INLINE void mingru_gates(const T* row, int n, int ch, float bz, float bx,
+                            float* z, float* cand) {
+  *z = sm_sigmoid(to_f(row[ch]) + bz);
+  const float u = to_f(row[n + ch]) + bx;
+  *cand = (u >= 0.f) ? u + 0.5f : sm_sigmoid(u);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mingru_chunk_reduce_kernel(
+    const T* __restrict__ zxg, const float* __restrict__ bias,
+    const int* __restrict__ chunks, int n, float* __restrict__ P,
+    float* __restrict__ Q) {
+  const int c = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= n) return;
+  const int t0 = chunks[3 * c + 1], cnt = chunks[3 * c + 2];
+  const float bz = bias[ch], bx = bias[n + ch];
+  float p = 1.f, q = 0.f;
+  for (int t = t0; t < t0 + cnt; ++t) {
+    float z, cand;
+    mingru_gates(zxg + (int64_t)t * 3 * n, n, ch, bz, bx, &z, &cand);
+    q = (1.0f - z) * q + z * cand;
+    p *= (1.0f - z);
+  }
+  P[(int64_t)c * n + ch] = p;
+  Q[(int64_t)c * n + ch] = q;
+}
+
+__global__ __launch_bounds__(256) void mingru_chunk_carry_kernel(
+    const float* __restrict__ P, const float* __restrict__ Q,
+    float* __restrict__ state, const int* __restrict__ chunk_cu,
+    const int* __restrict__ slots, int n, float* __restrict__ Sstart) {
+  const int b = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= n) return;
+  const int c0 = chunk_cu[b], c1 = chunk_cu[b + 1];
+  if (c1 == c0) return;
+  const int64_t slot = slots[b];
+  float S = state[slot * n + ch];
+  for (int c = c0; c < c1; ++c) {
+    Sstart[(int64_t)c * n + ch] = S;
+    S = P[(int64_t)c * n + ch] * S + Q[(int64_t)c * n + ch];
+  }
+  state[slot * n + ch] = S;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mingru_chunk_apply_kernel(
+    const T* __restrict__ zxg, const float* __restrict__ bias,
+    const int* __restrict__ chunks, const float* __restrict__ Sstart, int n,
+    T* __restrict__ out) {
+  const int c = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= n) return;
+  const int t0 = chunks[3 * c + 1], cnt = chunks[3 * c + 2];
+  const float bz = bias[ch], bx = bias[n + ch], bg = bias[2 * n + ch];
+  float S = Sstart[(int64_t)c * n + ch];
+  for (int t = t0; t < t0 + cnt; ++t) {
+    const T* row = zxg + (int64_t)t * 3 * n;
+    float z, cand;
+    mingru_gates(row, n, ch, bz, bx, &z, &cand);
+    S = (1.0f - z) * S + z * cand;
+    const float g = to_f(row[2 * n + ch]) + bg;
+    out[(int64_t)t * n + ch] = from_f<T>(S * (g * sm_sigmoid(g)));
+  }
+}
+
 // ------------------------------------------------------------- router
 // One workgroup per token: the waves share the experts' fp32 logits, then
 // one lane picks the top-k by repeated arg-max (ties: the lowest index) and
@@ -271,7 +344,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
 }  // namespace
 
 torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
-                          torch::Tensor cu, torch::Tensor slots) {
+                          torch::Tensor cu, torch::Tensor slots,
+                          c10::optional<torch::Tensor> chunks,
+                          c10::optional<torch::Tensor> chunk_cu) {
   SM_CHECK_CUDA(zxg); SM_CHECK_CUDA(bias); SM_CHECK_F32(bias);
   SM_CHECK_CUDA(state); SM_CHECK_F32(state);
   SM_CHECK_CUDA(cu); SM_CHECK_I32(cu); SM_CHECK_CUDA(slots); SM_CHECK_I32(slots);
@@ -283,6 +358,41 @@ torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor s
   auto out = torch::empty({T, n}, zxg.options());
   if (T == 0 || B == 0) return out;
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  if (chunks.has_value() && chunks->size(0) > 0) {
+    TORCH_CHECK(chunk_cu.has_value(), "mingru_scan: chunk_cu missing");
+    SM_CHECK_CUDA(*chunks); SM_CHECK_I32(*chunks); SM_CHECK_CUDA(*chunk_cu); SM_CHECK_I32(*chunk_cu);
+    TORCH_CHECK(chunks->dim() == 2 && chunks->size(1) == 3 && chunk_cu->numel() == B + 1,
+                "mingru_scan: chunk layout");
+    const int nc = chunks->size(0);
+    auto f32 = zxg.options().dtype(at::kFloat);
+    auto P = torch::empty({nc, n}, f32), Q = torch::empty({nc, n}, f32), S0 = torch::empty({nc, n}, f32);
+    dim3 gc(nc, SM_CDIV(n, 256)), gb(B, SM_CDIV(n, 256));
+    if (zxg.scalar_type() == at::kBFloat16)
+     hipLaunchKernelGGL(( mingru_chunk_reduce_kernel<bf16_t>), dim3(gc), dim3(256), 0, stream, 
+          reinterpret_cast<const bf16_t*>(zxg.data_ptr()), bias.data_ptr<float>(),
+          chunks->data_ptr<int>(), n, P.data_ptr<float>(), Q.data_ptr<float>());
+    else {
+      SM_CHECK_F32(zxg);
+     hipLaunchKernelGGL(( mingru_chunk_reduce_kernel<float>), dim3(gc), dim3(256), 0, stream, 
+          zxg.data_ptr<float>(), bias.data_ptr<float>(), chunks->data_ptr<int>(), n,
+          P.data_ptr<float>(), Q.data_ptr<float>());
+    }
+    SM_CHECK_LAUNCH();
+   hipLaunchKernelGGL(( mingru_chunk_carry_kernel), dim3(gb), dim3(256), 0, stream, 
+        P.data_ptr<float>(), Q.data_ptr<float>(), state.data_ptr<float>(),
+        chunk_cu->data_ptr<int>(), slots.data_ptr<int>(), n, S0.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    if (zxg.scalar_type() == at::kBFloat16)
+     hipLaunchKernelGGL(( mingru_chunk_apply_kernel<bf16_t>), dim3(gc), dim3(256), 0, stream, 
+          reinterpret_cast<const bf16_t*>(zxg.data_ptr()), bias.data_ptr<float>(),
+          chunks->data_ptr<int>(), S0.data_ptr<float>(), n, reinterpret_cast<bf16_t*>(out.data_ptr()));
+    else
+     hipLaunchKernelGGL(( mingru_chunk_apply_kernel<float>), dim3(gc), dim3(256), 0, stream, 
+          zxg.data_ptr<float>(), bias.data_ptr<float>(), chunks->data_ptr<int>(),
+          S0.data_ptr<float>(), n, out.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    return out;
+  }
   dim3 grid(B, SM_CDIV(n, 256));
   if (zxg.scalar_type() == at::kBFloat16)
    hipLaunchKernelGGL(( mingru_scan_kernel<bf16_t>), dim3(grid), dim3(256), 0, stream, 

@@ -86,9 +86,34 @@ def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                                      out_dtype)
 
 
-def mingru_scan(zxg, bias, state, cu, slots, out_dtype):
+SCAN_CHUNK = 64    # tokens per parallel chunk of a long row's recurrence
+
+
+def scan_chunks(row_lengths):
+    """Chunks of up to SCAN_CHUNK consecutive tokens per batch row, for the
+    parallel form of the recurrence: ([(row, first flat token, tokens)],
+    per-row chunk offsets). Empty when no row is longer than one chunk."""
+    if max(row_lengths, default=0) <= SCAN_CHUNK:
+        return [], []
+    chunks, cu, at = [], [0], 0
+    for b, n in enumerate(row_lengths):
+        for k in range(0, n, SCAN_CHUNK):
+            chunks.append((b, at + k, min(SCAN_CHUNK, n - k)))
+        cu.append(len(chunks))
+        at += n
+    return chunks, cu
+
+
+def mingru_scan(zxg, bias, state, cu, slots, out_dtype, chunks=None,
+                chunk_cu=None):
+    """``chunks``/``chunk_cu`` (from :func:`scan_chunks`) select the
+    three-pass chunk-parallel kernels; without them each (row, channel)
+    walks its tokens in order."""
     if zxg.is_cuda:
-        return _ext("mingru_scan").mingru_scan(zxg, bias, state, cu, slots)
+        if chunks is not None and chunks.numel() == 0:
+            chunks = chunk_cu = None
+        return _ext("mingru_scan").mingru_scan(zxg, bias, state, cu, slots,
+                                               chunks, chunk_cu)
     return R.mingru_scan(zxg, bias, state, cu, slots, out_dtype)
 
 

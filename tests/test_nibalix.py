@@ -424,6 +424,22 @@ def test_long_decode_keeps_state(dev):
     assert rel_err(O.forward(cfg, W, t2)[-1], want[-1]) > 1e-6
 
 
+def test_long_prompt_uses_chunked_scan(dev):
+    """Rows longer than one scan chunk take the chunk-parallel recurrence
+    (on the GPU); a long and a short row share the step."""
+    cfg = O.make_cfg([O.gru_layer(width=10, mlp=False), O.gru_layer(width=7, experts=2, top=1)],
+                     width=8, vocab=13, taps=3)
+    W, eng = build(cfg, dev, blocks=80, block_size=4)
+    a, b = toks(150, 13, seed=70), toks(5, 13, seed=71)
+    qa, qb = eng.open_sequence(), eng.open_sequence()
+    out = eng.step([(qa, a[:139]), (qb, b)], [list(range(139)), list(range(5))])
+    out2 = eng.step([(qa, a[139:])], [list(range(11))])
+    eng.close_sequence(qa)
+    eng.close_sequence(qb)
+    assert rel_err(torch.cat([out[:139], out2]), O.forward(cfg, W, a)) < tol(dev[1])
+    assert rel_err(out[139:], O.forward(cfg, W, b)) < tol(dev[1])
+
+
 def test_dirty_slot_and_pages_do_not_leak(dev):
     cfg = mixed_cfg()
     W, eng = build(cfg, dev, blocks=6, block_size=4, slots=1)
