@@ -215,24 +215,28 @@ SM_INLINE bf16v8 load8(const bf16_t* p, int valid, bool vec) {
   return v;
 }
 
-#define GG_BM 64
 #define GG_BK 64
 #define GG_LD 72   // padded LDS row (bf16 elements)
-template <int MODE>
-__global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
+// MT 16-row m-tiles per workgroup (rows BM = 16 MT) and NWV waves, each wave
+// owning 16 columns: <4, 4> is the 64x64 prompt tile; <1, 1> gives decode
+// batches (a few rows per expert) one wave per 16 columns, so that enough
+// workgroups stream the expert weights.
+template <int MODE, int MT, int NWV>
+__global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const int* __restrict__ src,
     const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
     int K, void* __restrict__ outp) {
-  __shared__ __attribute__((aligned(16))) bf16_t a_lds[GG_BM * GG_LD];
+  constexpr int BM = 16 * MT;
+  __shared__ __attribute__((aligned(16))) bf16_t a_lds[BM * GG_LD];
   // which expert / row range is this tile?
   int e = -1, row0 = 0, rows = 0, tiles = 0;
   for (int i = 0; i < E; ++i) {
     const int cnt = off[i + 1] - off[i];
-    const int nt = SM_CDIV(cnt, GG_BM);
+    const int nt = SM_CDIV(cnt, BM);
     if ((int)blockIdx.x < tiles + nt) {
       e = i;
-      row0 = off[i] + ((int)blockIdx.x - tiles) * GG_BM;
-      rows = min(GG_BM, off[i + 1] - row0);
+      row0 = off[i] + ((int)blockIdx.x - tiles) * BM;
+      rows = min(BM, off[i + 1] - row0);
       break;
     }
     tiles += nt;
@@ -241,30 +245,29 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63;
   const int lrow = l & 15, lk = l >> 4;
   const bool vec = (K % 8) == 0;
-  const int n = blockIdx.y * 64 + wave * 16 + lrow;     // this lane's B column
+  const int n = blockIdx.y * (16 * NWV) + wave * 16 + lrow;     // this lane's B column
   const int Nw = (MODE == 0) ? 2 * N : N;
   const bf16_t* Wg = W + ((int64_t)e * Nw + (n < N ? n : 0)) * K;
   const bf16_t* Wu = Wg + (int64_t)N * K;
-  f32x4 acc[4], acc2[4];
+  f32x4 acc[MT], acc2[MT];
   #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < MT; ++i) {
     acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc2[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   for (int k0 = 0; k0 < K; k0 += GG_BK) {
     __syncthreads();
-    #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-      const int r = pass * 32 + (tid >> 3), kc = (tid & 7) * 8;
-      bf16v8 v;
+    for (int v = tid; v < BM * 8; v += 64 * NWV) {
+      const int r = v >> 3, kc = (v & 7) * 8;
+      bf16v8 val;
       if (r < rows) {
         const int64_t arow = (MODE == 0) ? src[row0 + r] : (row0 + r);
-        v = load8(A + arow * K + k0 + kc, K - (k0 + kc), vec);
+        val = load8(A + arow * K + k0 + kc, K - (k0 + kc), vec);
       } else {
         #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = (__bf16)0.0f;
+        for (int j = 0; j < 8; ++j) val[j] = (__bf16)0.0f;
       }
-      *reinterpret_cast<bf16v8*>(a_lds + r * GG_LD + kc) = v;
+      *reinterpret_cast<bf16v8*>(a_lds + r * GG_LD + kc) = val;
     }
     __syncthreads();
     #pragma unroll
@@ -276,7 +279,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
       bg = load8(Wg + kk, valid, vec);
       if (MODE == 0) bu = load8(Wu + kk, valid, vec);
       #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) {
         const bf16v8 a = *reinterpret_cast<const bf16v8*>(
             a_lds + (mt * 16 + lrow) * GG_LD + ks * 32 + lk * 8);
         acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bg, acc[mt], 0, 0, 0);
@@ -285,15 +288,14 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
       }
     }
   }
-  const int col = blockIdx.y * 64 + wave * 16 + lrow;
-  if (col >= N) return;
+  if (n >= N) return;
   #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
     #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const int r = mt * 16 + lk * 4 + rr;
       if (r < rows) {
-        const int64_t o = (int64_t)(row0 + r) * N + col;
+        const int64_t o = (int64_t)(row0 + r) * N + n;
         if (MODE == 0) {
           const float g = acc[mt][rr];
           reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(g * sm_sigmoid(g) * acc2[mt][rr]);
@@ -468,17 +470,29 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
   auto y = torch::empty({M, D}, out.options());
   if (h.scalar_type() == at::kBFloat16) {
     auto act = torch::empty({M, ff}, h.options());
-    const int row_tiles = SM_CDIV(M, GG_BM) + E;
-   hipLaunchKernelGGL(( moe_gemm_bf16_kernel<0>), dim3(dim3(row_tiles, SM_CDIV(ff, 64))), dim3(256), 0, stream, 
-        reinterpret_cast<const bf16_t*>(h.data_ptr()), src.data_ptr<int>(),
-        reinterpret_cast<const bf16_t*>(exp_gu.data_ptr()), off.data_ptr<int>(), E, ff, D,
-        act.data_ptr());
-    SM_CHECK_LAUNCH();
-   hipLaunchKernelGGL(( moe_gemm_bf16_kernel<1>), dim3(dim3(row_tiles, SM_CDIV(D, 64))), dim3(256), 0, stream, 
-        reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr,
-        reinterpret_cast<const bf16_t*>(exp_down.data_ptr()), off.data_ptr<int>(), E, D, ff,
-        y.data_ptr());
-    SM_CHECK_LAUNCH();
+    const bf16_t* hp = reinterpret_cast<const bf16_t*>(h.data_ptr());
+    const bf16_t* gup = reinterpret_cast<const bf16_t*>(exp_gu.data_ptr());
+    const bf16_t* dnp = reinterpret_cast<const bf16_t*>(exp_down.data_ptr());
+    if (M <= 16 * E) {
+      // a few rows per expert (decoding): 16-row tiles, one wave per 16 columns
+      const int row_tiles = SM_CDIV(M, 16) + E;
+     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<0, 1, 1>), dim3(dim3(row_tiles, SM_CDIV(ff, 16))), dim3(64), 0, stream, 
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr());
+      SM_CHECK_LAUNCH();
+     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<1, 1, 1>), dim3(dim3(row_tiles, SM_CDIV(D, 16))), dim3(64), 0, stream, 
+          reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
+          D, ff, y.data_ptr());
+      SM_CHECK_LAUNCH();
+    } else {
+      const int row_tiles = SM_CDIV(M, 64) + E;
+     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<0, 4, 4>), dim3(dim3(row_tiles, SM_CDIV(ff, 64))), dim3(256), 0, stream, 
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr());
+      SM_CHECK_LAUNCH();
+     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<1, 4, 4>), dim3(dim3(row_tiles, SM_CDIV(D, 64))), dim3(256), 0, stream, 
+          reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
+          D, ff, y.data_ptr());
+      SM_CHECK_LAUNCH();
+    }
   } else {
     SM_CHECK_F32(h);
     auto act = torch::empty({M, ff}, h.options());

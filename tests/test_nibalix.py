@@ -292,11 +292,11 @@ def test_mingru_scan_portions_and_slots(dev):
     assert (pre[:, n:2 * n] + bias[n:2 * n] >= 0).any() and (pre[:, n:2 * n] + bias[n:2 * n] < 0).any()
 
 
-@pytest.mark.parametrize("experts,top,D,ff", [(5, 2, 16, 10), (4, 1, 16, 10), (3, 3, 16, 10),
-                                              (9, 4, 16, 10), (4, 2, 104, 72), (3, 2, 33, 70)])
-def test_moe(dev, experts, top, D, ff):
+@pytest.mark.parametrize("experts,top,D,ff,T", [(5, 2, 16, 10, 70), (4, 1, 16, 10, 70), (3, 3, 16, 10, 70),
+                                                (9, 4, 16, 10, 70), (4, 2, 104, 72, 70), (3, 2, 33, 70, 70),
+                                                (4, 2, 104, 72, 5), (6, 3, 40, 24, 17), (2, 1, 16, 10, 1)])
+def test_moe(dev, experts, top, D, ff, T):
     device, dtype = dev
-    T = 70
     cfg = O.make_cfg([O.gru_layer(width=4, experts=experts, top=top, ff=ff)], width=D)
     Wf = O.random_weights(cfg, 7)
     W = {k: v.double() for k, v in Wf.items()}
@@ -309,7 +309,7 @@ def test_moe(dev, experts, top, D, ff):
     want = torch.stack([O.moe(r.double(), W, "l0.mlp.", cfg["layers"][0]["mlp"]) for r in h])
     assert rel_err(got, want) < tol(dtype)
     assert rel_err(wts.sum(-1), torch.ones(T)) < 1e-5
-    assert len(set(idx.flatten().tolist())) == experts          # every expert is used
+    assert T < 40 or len(set(idx.flatten().tolist())) == experts    # every expert is used
 
 
 def test_router_tie_takes_lowest_index(dev):
