@@ -416,6 +416,165 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
   }
 }
 
+
+// ---- prompt tiles, all on MFMA: four waves share one tile of up to 16
+// queries of one head. Each 32-key block of the cache is staged in LDS once;
+// every wave forms the block's scores and fp32 softmax weights (the same in
+// all four), then takes every fourth 16-wide slice of the latent axis of the
+// weighted sum: O[q, f] += sum_k P[q, k] C[k, f] as MFMA with the weights
+// split into two bf16 terms (p = hi + lo, |p - hi - lo| <= 2^-17 p), so the
+// fp32 weights keep 16+ bits against the bf16 latents; accumulation is fp32.
+#define LC_NT 8      // latent slices per wave: kv_rank <= 4 * 8 * 16
+__global__ __launch_bounds__(256) void latent_attention_coop_kernel(
+    const bf16_t* __restrict__ q_lat, const float* __restrict__ q_rot,
+    const bf16_t* __restrict__ cache, const int* __restrict__ block_tables,
+    int max_nb, int block_size, const int* __restrict__ tiles,
+    const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
+    float scale, bf16_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int W = r + rd;
+  const int Wp = ((W + 31) / 32) * 32 + 8;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const int lrow = l & 15, lk = l >> 4;
+  bf16_t* q_lds = reinterpret_cast<bf16_t*>(smem);                 // [16][Wp]
+  bf16_t* c_lds = q_lds + LT_TQ * Wp;                               // [32][Wp]
+  float* p_lds = reinterpret_cast<float*>(c_lds + LT_KB * Wp) + wave * (LT_TQ * LT_KB);
+
+  const int tile = blockIdx.x, hd = blockIdx.y;
+  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
+  const int p0 = positions[t0], plast = p0 + nq - 1;
+  const int lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+  const int nkeys = plast - lo + 1;
+  const int nblk = (nkeys + LT_KB - 1) / LT_KB;
+  const int* bt = block_tables + (int64_t)b * max_nb;
+  const bool vec = (W % 8) == 0;
+
+  // queries [latent | rotated], zero padded; key block area zeroed once
+  for (int i = threadIdx.x; i < LT_TQ * Wp; i += blockDim.x) {
+    const int q = i / Wp, k = i % Wp;
+    float v = 0.f;
+    if (q < nq) {
+      if (k < r) v = to_f(q_lat[((int64_t)hd * Tn + t0 + q) * r + k]);
+      else if (k < W) v = q_rot[((int64_t)(t0 + q) * H + hd) * rd + (k - r)];
+    }
+    q_lds[i] = __float2bfloat16(v);
+  }
+  for (int i = threadIdx.x; i < LT_KB * Wp; i += blockDim.x) c_lds[i] = __float2bfloat16(0.f);
+
+  float m[4], lsum[4];
+  #pragma unroll
+  for (int rr = 0; rr < 4; ++rr) { m[rr] = -INFINITY; lsum[rr] = 0.f; }
+  f32x4_t acc[LC_NT];
+  #pragma unroll
+  for (int i = 0; i < LC_NT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int KS = (W + 31) / 32;
+  const int ntiles_f = (r + 15) / 16;
+
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int j0 = lo + kb * LT_KB;
+    const int nk = min(LT_KB, nkeys - kb * LT_KB);
+    __syncthreads();                       // the previous block is fully consumed
+    if (vec) {
+      const int w8 = W / 8;
+      for (int i = threadIdx.x; i < nk * w8; i += blockDim.x) {
+        const int kk = i / w8, k = (i % w8) * 8;
+        const int j = j0 + kk;
+        const int64_t row = (int64_t)bt[j / block_size] * block_size + j % block_size;
+        *reinterpret_cast<bf16v8_t*>(c_lds + kk * Wp + k) =
+            *reinterpret_cast<const bf16v8_t*>(cache + row * W + k);
+      }
+    } else {
+      for (int i = threadIdx.x; i < nk * W; i += blockDim.x) {
+        const int kk = i / W, k = i % W;
+        const int j = j0 + kk;
+        const int64_t row = (int64_t)bt[j / block_size] * block_size + j % block_size;
+        c_lds[kk * Wp + k] = cache[row * W + k];
+      }
+    }
+    __syncthreads();
+    // scores of the 32 keys (two 16-key MFMA tiles), same in every wave
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < KS; ++ks) {
+      const int f0 = ks * 32 + lk * 8;
+      const bf16v8_t a = *reinterpret_cast<const bf16v8_t*>(q_lds + lrow * Wp + f0);
+      const bf16v8_t b0 = *reinterpret_cast<const bf16v8_t*>(c_lds + lrow * Wp + f0);
+      const bf16v8_t b1 = *reinterpret_cast<const bf16v8_t*>(c_lds + (16 + lrow) * Wp + f0);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b0, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, s1, 0, 0, 0);
+    }
+    float cr[4];
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int q = lk * 4 + rr;
+      const int pq = p0 + q;
+      const int ja = j0 + lrow, jb = j0 + 16 + lrow;
+      const bool oka = q < nq && ja <= pq && (window <= 0 || pq - ja < window);
+      const bool okb = q < nq && jb <= pq && (window <= 0 || pq - jb < window);
+      const float sa = oka ? s0[rr] * scale : -INFINITY;
+      const float sb = okb ? s1[rr] * scale : -INFINITY;
+      float bm = fmaxf(sa, sb);
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, SM_WAVE));
+      const float mn = fmaxf(m[rr], bm);
+      const float c = (mn == -INFINITY) ? 1.0f : expf(m[rr] - mn);
+      const float pa = oka ? expf(sa - mn) : 0.f;
+      const float pb = okb ? expf(sb - mn) : 0.f;
+      float ps = pa + pb;
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, SM_WAVE);
+      lsum[rr] = lsum[rr] * c + ps;
+      m[rr] = mn;
+      cr[rr] = c;
+      p_lds[q * LT_KB + lrow] = pa;
+      p_lds[q * LT_KB + 16 + lrow] = pb;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    // weights as the A operand: row = query lrow, k = keys lk*8 .. +7
+    bf16v8_t a_hi, a_lo;
+    #pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float pv = p_lds[lrow * LT_KB + lk * 8 + j];
+      const __bf16 hi = (__bf16)pv;
+      a_hi[j] = hi;
+      a_lo[j] = (__bf16)(pv - (float)hi);
+    }
+    #pragma unroll
+    for (int i = 0; i < LC_NT; ++i) {
+      const int nt = wave + 4 * i;
+      if (nt < ntiles_f) {
+        const int f = nt * 16 + lrow;         // padding columns of c_lds are zero
+        bf16v8_t bc;
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const bf16_t v = c_lds[(lk * 8 + j) * Wp + f];
+          bc[j] = *reinterpret_cast<const __bf16*>(&v);
+        }
+        f32x4_t a4 = acc[i];
+        #pragma unroll
+        for (int rr = 0; rr < 4; ++rr) a4[rr] *= cr[rr];
+        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bc, a4, 0, 0, 0);
+        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bc, a4, 0, 0, 0);
+        acc[i] = a4;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  #pragma unroll
+  for (int i = 0; i < LC_NT; ++i) {
+    const int nt = wave + 4 * i;
+    const int f = nt * 16 + lrow;
+    if (nt < ntiles_f && f < r) {
+      #pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int q = lk * 4 + rr;
+        if (q < nq)
+          out[((int64_t)hd * Tn + t0 + q) * r + f] = __float2bfloat16(acc[i][rr] / lsum[rr]);
+      }
+    }
+  }
+}
+
 // Merge the key splits of one (token, head): out = sum_z acc_z e^(m_z - M) / L.
 __global__ __launch_bounds__(256) void latent_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
@@ -517,6 +676,20 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     // decode-only batches (one query per row): a tile is one token with up
     // to 16 of its heads, and four waves split its keys
     const bool heads = max_tile_queries == 1 && H > 1;
+    if (!heads && max_tile_queries > 4) {
+      // prompt portions: the four-wave all-MFMA kernel
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * Wp * 2 + 4 * LT_TQ * LT_KB * 4;
+      if (ldsc <= 64 * 1024) {
+       hipLaunchKernelGGL(( latent_attention_coop_kernel), dim3(dim3(ntiles, H)), dim3(256), ldsc, stream, 
+            reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
+            reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
+            (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),
+            positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
+            reinterpret_cast<bf16_t*>(out.data_ptr()));
+        SM_CHECK_LAUNCH();
+        return out;
+      }
+    }
     const int NW = (heads || (max_tile_queries <= 4 && (int64_t)ntiles * H < 4096)) ? 4 : 1;
     const int nq_cap = heads ? LT_TQ : (int)max_tile_queries;
     size_t lds2 = (size_t)LT_TQ * Wp * 2 + (size_t)NW * (LT_TQ * LT_KB + LT_KB + LT_TQ) * 4 +

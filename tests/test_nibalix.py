@@ -222,15 +222,18 @@ def test_attention_matches_oracle_scores(dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("r,rd,window,lens", [(128, 32, 100, [300, 1, 37, 2]),
-                                              (104, 24, 45, [70, 16, 17, 1]),
-                                              (320, 64, 0, [50, 3]),
-                                              (72, 20, 33, [1, 1, 1, 1, 1])])
-def test_tiled_attention_kernel_against_plain_op(r, rd, window, lens):
+@pytest.mark.parametrize("r,rd,window,lens,H", [(128, 32, 100, [300, 1, 37, 2], 3),
+                                                (104, 24, 45, [70, 16, 17, 1], 3),
+                                                (320, 64, 0, [50, 3], 2),
+                                                (72, 20, 33, [1, 1, 1, 1, 1], 3),
+                                                (64, 8, 500, [1, 1, 1], 20),
+                                                (512, 64, 120, [1, 1], 16),
+                                                (33, 6, 7, [40, 1], 1)])
+def test_tiled_attention_kernel_against_plain_op(r, rd, window, lens, H):
     """bf16 MFMA tiles (several tiles per row, ragged last tile, four-wave
     key split for decode-only batches) against the fp32 torch form."""
     from distrl_llm_amd.ops import seqmix_reference as R
-    H, bs = 3, 16
+    bs = 16
     g = torch.Generator().manual_seed(r)
     ctx = [n + 150 for n in lens]                       # tokens before this step
     nblk = [(c + bs - 1) // bs for c in ctx]
