@@ -424,12 +424,17 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
 // split into two bf16 terms (p = hi + lo, |p - hi - lo| <= 2^-17 p), so the
 // fp32 weights keep 16+ bits against the bf16 latents; accumulation is fp32.
 #define LC_NT 8      // latent slices per wave: kv_rank <= 4 * 8 * 16
+// HEADS: rows are up to 16 heads of one token (decoding); blockIdx.z then
+// takes a share of the key blocks and leaves (max, sum, unnormalised sum)
+// for latent_combine when ksplit > 1.
+template <bool HEADS>
 __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     const bf16_t* __restrict__ q_lat, const float* __restrict__ q_rot,
     const bf16_t* __restrict__ cache, const int* __restrict__ block_tables,
     int max_nb, int block_size, const int* __restrict__ tiles,
     const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
-    float scale, bf16_t* __restrict__ out) {
+    float scale, bf16_t* __restrict__ out, int ksplit,
+    float* __restrict__ part_acc, float* __restrict__ part_ml) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int W = r + rd;
   const int Wp = ((W + 31) / 32) * 32 + 8;
@@ -439,9 +444,11 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
   bf16_t* c_lds = q_lds + LT_TQ * Wp;                               // [32][Wp]
   float* p_lds = reinterpret_cast<float*>(c_lds + LT_KB * Wp) + wave * (LT_TQ * LT_KB);
 
-  const int tile = blockIdx.x, hd = blockIdx.y;
-  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
-  const int p0 = positions[t0], plast = p0 + nq - 1;
+  const int tile = blockIdx.x;
+  const int hd = HEADS ? blockIdx.y * LT_TQ : blockIdx.y;
+  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1];
+  const int nq = HEADS ? min(LT_TQ, H - hd) : tiles[3 * tile + 2];
+  const int p0 = positions[t0], plast = HEADS ? p0 : p0 + nq - 1;
   const int lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
   const int nkeys = plast - lo + 1;
   const int nblk = (nkeys + LT_KB - 1) / LT_KB;
@@ -453,8 +460,9 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     const int q = i / Wp, k = i % Wp;
     float v = 0.f;
     if (q < nq) {
-      if (k < r) v = to_f(q_lat[((int64_t)hd * Tn + t0 + q) * r + k]);
-      else if (k < W) v = q_rot[((int64_t)(t0 + q) * H + hd) * rd + (k - r)];
+      const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+      if (k < r) v = to_f(q_lat[((int64_t)hq * Tn + tq) * r + k]);
+      else if (k < W) v = q_rot[((int64_t)tq * H + hq) * rd + (k - r)];
     }
     q_lds[i] = __float2bfloat16(v);
   }
@@ -469,7 +477,10 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
   const int KS = (W + 31) / 32;
   const int ntiles_f = (r + 15) / 16;
 
-  for (int kb = 0; kb < nblk; ++kb) {
+  const int kb_lo = (int)(((int64_t)nblk * blockIdx.z) / ksplit);
+  const int kb_hi = (int)(((int64_t)nblk * (blockIdx.z + 1)) / ksplit);
+  if (kb_hi == kb_lo) __syncthreads();     // the LDS fills above, before any exit
+  for (int kb = kb_lo; kb < kb_hi; ++kb) {
     const int j0 = lo + kb * LT_KB;
     const int nk = min(LT_KB, nkeys - kb * LT_KB);
     __syncthreads();                       // the previous block is fully consumed
@@ -505,7 +516,7 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const int q = lk * 4 + rr;
-      const int pq = p0 + q;
+      const int pq = HEADS ? p0 : p0 + q;
       const int ja = j0 + lrow, jb = j0 + 16 + lrow;
       const bool oka = q < nq && ja <= pq && (window <= 0 || pq - ja < window);
       const bool okb = q < nq && jb <= pq && (window <= 0 || pq - jb < window);
@@ -559,6 +570,17 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   }
+  if (ksplit > 1 && wave == 0 && lrow == 0) {
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int q = lk * 4 + rr;
+      if (q < nq) {
+        const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+        part_ml[(((int64_t)tq * H + hq) * ksplit + blockIdx.z) * 2] = m[rr];
+        part_ml[(((int64_t)tq * H + hq) * ksplit + blockIdx.z) * 2 + 1] = lsum[rr];
+      }
+    }
+  }
   #pragma unroll
   for (int i = 0; i < LC_NT; ++i) {
     const int nt = wave + 4 * i;
@@ -567,8 +589,13 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
       #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int q = lk * 4 + rr;
-        if (q < nq)
-          out[((int64_t)hd * Tn + t0 + q) * r + f] = __float2bfloat16(acc[i][rr] / lsum[rr]);
+        if (q < nq) {
+          const int tq = HEADS ? t0 : t0 + q, hq = HEADS ? hd + q : hd;
+          if (ksplit > 1)
+            part_acc[(((int64_t)tq * H + hq) * ksplit + blockIdx.z) * r + f] = acc[i][rr];
+          else
+            out[((int64_t)hq * Tn + tq) * r + f] = __float2bfloat16(acc[i][rr] / lsum[rr]);
+        }
       }
     }
   }
@@ -679,13 +706,44 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
       // prompt portions: the four-wave all-MFMA kernel
       const size_t ldsc = (size_t)(LT_TQ + LT_KB) * Wp * 2 + 4 * LT_TQ * LT_KB * 4;
       if (ldsc <= 64 * 1024) {
-        latent_attention_coop_kernel<<<dim3(ntiles, H), 256, ldsc, stream>>>(
+        latent_attention_coop_kernel<false><<<dim3(ntiles, H), 256, ldsc, stream>>>(
             reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
             reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
             (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),
             positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
-            reinterpret_cast<bf16_t*>(out.data_ptr()));
+            reinterpret_cast<bf16_t*>(out.data_ptr()), 1, nullptr, nullptr);
         SM_CHECK_LAUNCH();
+        return out;
+      }
+    }
+    if (heads) {
+      // decoding: one token x up to 16 heads per workgroup, the key blocks
+      // spread over blockIdx.z, merged by latent_combine
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * Wp * 2 + 4 * LT_TQ * LT_KB * 4;
+      if (ldsc <= 64 * 1024) {
+        const int64_t groups = (int64_t)ntiles * SM_CDIV(H, LT_TQ);
+        int ks = (int)std::min<int64_t>(32, std::max<int64_t>(1, 1024 / groups));
+        if (window > 0) ks = (int)std::min<int64_t>(ks, SM_CDIV(window, LT_KB) + 1);
+        torch::Tensor pa, pm;
+        float *pap = nullptr, *pmp = nullptr;
+        if (ks > 1) {
+          pa = torch::empty({T, H, ks, r}, q_rot.options());
+          pm = torch::empty({T, H, ks, 2}, q_rot.options());
+          pap = pa.data_ptr<float>();
+          pmp = pm.data_ptr<float>();
+        }
+        latent_attention_coop_kernel<true><<<dim3(ntiles, SM_CDIV(H, LT_TQ), ks), 256, ldsc, stream>>>(
+            reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
+            reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
+            (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),
+            positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
+            reinterpret_cast<bf16_t*>(out.data_ptr()), ks, pap, pmp);
+        SM_CHECK_LAUNCH();
+        if (ks > 1) {
+          latent_combine_kernel<<<(int)(T * H), 256, 0, stream>>>(
+              pap, pmp, (int)T, H, r, ks, reinterpret_cast<bf16_t*>(out.data_ptr()));
+          SM_CHECK_LAUNCH();
+        }
         return out;
       }
     }
