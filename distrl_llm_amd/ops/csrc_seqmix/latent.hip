@@ -424,6 +424,10 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
 // split into two bf16 terms (p = hi + lo, |p - hi - lo| <= 2^-17 p), so the
 // fp32 weights keep 16+ bits against the bf16 latents; accumulation is fp32.
 #define LC_NT 8      // latent slices per wave: kv_rank <= 4 * 8 * 16
+// LDS row length (bf16) of the staged queries / key block: a multiple of 8
+// (16-byte pieces) that is 16 mod 64, so that neighbouring rows start 8
+// banks apart and the four lane groups of a weighted-sum gather do not collide
+#define LC_ROW(W) ((((W) + 31) / 32) * 32 + ((((W) + 31) / 32) % 2 ? 48 : 16))
 // HEADS: rows are up to 16 heads of one token (decoding); blockIdx.z then
 // takes a share of the key blocks and leaves (max, sum, unnormalised sum)
 // for latent_combine when ksplit > 1.
@@ -437,7 +441,7 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int W = r + rd;
-  const int Wp = ((W + 31) / 32) * 32 + 8;
+  const int Wp = LC_ROW(W);
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
   const int lrow = l & 15, lk = l >> 4;
   bf16_t* q_lds = reinterpret_cast<bf16_t*>(smem);                 // [16][Wp]
@@ -540,11 +544,13 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xc07f);
-    // weights as the A operand: row = query lrow, k = keys lk*8 .. +7
+    // weights as the A operand: row = query lrow; the MFMA's k index runs
+    // over the keys lk + 4 j (any order works as long as A and B agree; this
+    // one puts the four lane groups on neighbouring LDS rows of the block)
     bf16v8_t a_hi, a_lo;
     #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float pv = p_lds[lrow * LT_KB + lk * 8 + j];
+      const float pv = p_lds[lrow * LT_KB + lk + 4 * j];
       const __bf16 hi = (__bf16)pv;
       a_hi[j] = hi;
       a_lo[j] = (__bf16)(pv - (float)hi);
@@ -557,7 +563,7 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
         bf16v8_t bc;
         #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const bf16_t v = c_lds[(lk * 8 + j) * Wp + f];
+          const bf16_t v = c_lds[(lk + 4 * j) * Wp + f];
           bc[j] = *reinterpret_cast<const __bf16*>(&v);
         }
         f32x4_t a4 = acc[i];
@@ -704,7 +710,7 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     const bool heads = max_tile_queries == 1 && H > 1;
     if (!heads && max_tile_queries > 4) {
       // prompt portions: the four-wave all-MFMA kernel
-      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * Wp * 2 + 4 * LT_TQ * LT_KB * 4;
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 4 * LT_TQ * LT_KB * 4;
       if (ldsc <= 64 * 1024) {
         latent_attention_coop_kernel<false><<<dim3(ntiles, H), 256, ldsc, stream>>>(
             reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
@@ -719,7 +725,7 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     if (heads) {
       // decoding: one token x up to 16 heads per workgroup, the key blocks
       // spread over blockIdx.z, merged by latent_combine
-      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * Wp * 2 + 4 * LT_TQ * LT_KB * 4;
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 4 * LT_TQ * LT_KB * 4;
       if (ldsc <= 64 * 1024) {
         const int64_t groups = (int64_t)ntiles * SM_CDIV(H, LT_TQ);
         int ks = (int)std::min<int64_t>(32, std::max<int64_t>(1, 1024 / groups));

@@ -307,6 +307,80 @@ __global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
   }
 }
 
+// Decode batches (a few rows per expert): one 16-row x 16-column tile per
+// workgroup, the K axis dealt out to the four waves in 32-wide steps (every
+// lane reads its A and B fragments straight from memory: no LDS, no barrier
+// in the loop, four times the loads in flight), partial tiles summed
+// through LDS in a fixed order.
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_gemm_bf16_splitk_kernel(
+    const bf16_t* __restrict__ A, const int* __restrict__ src,
+    const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
+    int K, void* __restrict__ outp) {
+  __shared__ float red[3][64][8];
+  int e = -1, row0 = 0, rows = 0, tiles = 0;
+  for (int i = 0; i < E; ++i) {
+    const int cnt = off[i + 1] - off[i];
+    const int nt = SM_CDIV(cnt, 16);
+    if ((int)blockIdx.x < tiles + nt) {
+      e = i;
+      row0 = off[i] + ((int)blockIdx.x - tiles) * 16;
+      rows = min(16, off[i + 1] - row0);
+      break;
+    }
+    tiles += nt;
+  }
+  if (e < 0) return;                       // uniform over the workgroup
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const int lrow = l & 15, lk = l >> 4;
+  const bool vec = (K % 8) == 0;
+  const int n = blockIdx.y * 16 + lrow;
+  const int Nw = (MODE == 0) ? 2 * N : N;
+  const bf16_t* Wg = W + ((int64_t)e * Nw + (n < N ? n : 0)) * K;
+  const bf16_t* Wu = Wg + (int64_t)N * K;
+  const int64_t arow = (lrow < rows) ? ((MODE == 0) ? src[row0 + lrow] : (row0 + lrow)) : -1;
+  const bf16_t* ap = A + (arow < 0 ? 0 : arow) * K;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  #pragma unroll 4
+  for (int k0 = wave * 32; k0 < K; k0 += 128) {      // uniform within a wave
+    const int kk = k0 + lk * 8;
+    const bf16v8 a = load8(ap + kk, arow < 0 ? 0 : K - kk, vec);
+    const int valid = (n < N) ? K - kk : 0;
+    const bf16v8 bg = load8(Wg + kk, valid, vec);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bg, acc, 0, 0, 0);
+    if (MODE == 0) {
+      const bf16v8 bu = load8(Wu + kk, valid, vec);
+      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bu, acc2, 0, 0, 0);
+    }
+  }
+  if (wave > 0) {
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      red[wave - 1][l][rr] = acc[rr];
+      red[wave - 1][l][4 + rr] = acc2[rr];
+    }
+  }
+  __syncthreads();
+  if (wave > 0 || n >= N) return;
+  #pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    float g = acc[rr], u = acc2[rr];
+    #pragma unroll
+    for (int w = 0; w < 3; ++w) {
+      g += red[w][l][rr];
+      u += red[w][l][4 + rr];
+    }
+    const int r = lk * 4 + rr;
+    if (r < rows) {
+      const int64_t o = (int64_t)(row0 + r) * N + n;
+      if (MODE == 0)
+        reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(g * sm_sigmoid(g) * u);
+      else
+        reinterpret_cast<float*>(outp)[o] = g;
+    }
+  }
+}
+
 // ------------------------------------------------- grouped GEMM, fp32
 // One thread per output element; the expert of a row by scanning off[].
 template <int MODE>
@@ -474,12 +548,12 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
     const bf16_t* gup = reinterpret_cast<const bf16_t*>(exp_gu.data_ptr());
     const bf16_t* dnp = reinterpret_cast<const bf16_t*>(exp_down.data_ptr());
     if (M <= 16 * E) {
-      // a few rows per expert (decoding): 16-row tiles, one wave per 16 columns
+      // a few rows per expert (decoding): 16x16 tiles, K split over four waves
       const int row_tiles = SM_CDIV(M, 16) + E;
-     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<0, 1, 1>), dim3(dim3(row_tiles, SM_CDIV(ff, 16))), dim3(64), 0, stream, 
+     hipLaunchKernelGGL(( moe_gemm_bf16_splitk_kernel<0>), dim3(dim3(row_tiles, SM_CDIV(ff, 16))), dim3(256), 0, stream, 
           hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr());
       SM_CHECK_LAUNCH();
-     hipLaunchKernelGGL(( moe_gemm_bf16_kernel<1, 1, 1>), dim3(dim3(row_tiles, SM_CDIV(D, 16))), dim3(64), 0, stream, 
+     hipLaunchKernelGGL(( moe_gemm_bf16_splitk_kernel<1>), dim3(dim3(row_tiles, SM_CDIV(D, 16))), dim3(256), 0, stream, 
           reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
           D, ff, y.data_ptr());
       SM_CHECK_LAUNCH();
