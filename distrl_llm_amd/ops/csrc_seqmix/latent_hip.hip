@@ -484,29 +484,37 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
 
   const int kb_lo = (int)(((int64_t)nblk * blockIdx.z) / ksplit);
   const int kb_hi = (int)(((int64_t)nblk * (blockIdx.z + 1)) / ksplit);
+  // cache rows of a block's 32 keys: looked up by 32 lanes one block ahead,
+  // so the copy below does not chain a block-table load before every piece
+  __shared__ int krow[LT_KB];
+  auto key_rows = [&](int kb2) {
+    if (threadIdx.x < LT_KB) {
+      const int j = min(lo + kb2 * LT_KB + (int)threadIdx.x, plast);
+      krow[threadIdx.x] = bt[j / block_size] * block_size + j % block_size;
+    }
+  };
+  if (kb_lo < kb_hi) key_rows(kb_lo);
   if (kb_hi == kb_lo) __syncthreads();     // the LDS fills above, before any exit
   for (int kb = kb_lo; kb < kb_hi; ++kb) {
-    const int j0 = lo + kb * LT_KB;
     const int nk = min(LT_KB, nkeys - kb * LT_KB);
     __syncthreads();                       // the previous block is fully consumed
     if (vec) {
       const int w8 = W / 8;
+      #pragma unroll 4
       for (int i = threadIdx.x; i < nk * w8; i += blockDim.x) {
         const int kk = i / w8, k = (i % w8) * 8;
-        const int j = j0 + kk;
-        const int64_t row = (int64_t)bt[j / block_size] * block_size + j % block_size;
         *reinterpret_cast<bf16v8_t*>(c_lds + kk * Wp + k) =
-            *reinterpret_cast<const bf16v8_t*>(cache + row * W + k);
+            *reinterpret_cast<const bf16v8_t*>(cache + (int64_t)krow[kk] * W + k);
       }
     } else {
       for (int i = threadIdx.x; i < nk * W; i += blockDim.x) {
         const int kk = i / W, k = i % W;
-        const int j = j0 + kk;
-        const int64_t row = (int64_t)bt[j / block_size] * block_size + j % block_size;
-        c_lds[kk * Wp + k] = cache[row * W + k];
+        c_lds[kk * Wp + k] = cache[(int64_t)krow[kk] * W + k];
       }
     }
     __syncthreads();
+    if (kb + 1 < kb_hi) key_rows(kb + 1);  // read again only after the next barrier
+    const int j0 = lo + kb * LT_KB;
     // scores of the 32 keys (two 16-key MFMA tiles), same in every wave
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
     for (int ks = 0; ks < KS; ++ks) {
