@@ -308,8 +308,11 @@ class HybridEngine:
         h32, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt)
         last = S.num_layers - 1
         for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
-            hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i], cu,
-                                    meta["tok_seq"], slots, dt)
+            if S.conv_taps:
+                hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i], cu,
+                                        meta["tok_seq"], slots, dt)
+            else:
+                hm = hb
             gates = F.linear(hb, L.gate_w)
             m = ls.mixer
             if isinstance(m, LatentAttentionSpec):

@@ -66,7 +66,7 @@ class StateSlotPool:
     def __init__(self, spec: HybridSpec, num_slots: int, device):
         self.num_slots = num_slots
         self.scratch_slot = num_slots     # never handed out (padding rows)
-        D, k = spec.width, spec.conv_taps - 1
+        D, k = spec.width, max(spec.conv_taps - 1, 0)
         # conv tails: one tensor per layer, [slots + 1, taps-1, width] fp32
         self.tails: List[torch.Tensor] = [
             torch.zeros(num_slots + 1, k, D, dtype=torch.float32, device=device)

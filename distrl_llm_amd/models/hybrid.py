@@ -105,10 +105,13 @@ def nibalix_spec_from_config(cfg: dict, name: str = "nibalix") -> HybridSpec:
             mixer = LatentAttentionSpec(
                 heads=int(mc["heads"]), dim=int(mc["dim"]),
                 rot_dim=int(mc["rot_dim"]), vdim=int(mc["vdim"]),
-                kv_rank=int(mc["kv_rank"]), scale=float(mc["scale"]),
-                rope_base=float(rot.get("base", 10000.0)),
-                rope_dims=int(rot.get("dims", mc["rot_dim"])),
-                window=int((mc.get("mask") or {}).get("size", 0)),
+                kv_rank=int(mc["kv_rank"]),
+                scale=float(mc["scale"] if mc.get("scale") is not None
+                            else (int(mc["dim"]) + int(mc["rot_dim"])) ** -0.5),
+                rope_base=float(rot.get("base") or 10000.0),
+                rope_dims=int(rot["dims"] if rot.get("dims") is not None
+                              else mc["rot_dim"]),
+                window=int((mc.get("mask") or {}).get("size") or 0),
                 kv_from=(int(mc["kv_from"]) if mc.get("kv_from") is not None
                          else None))
             if mixer.rope_dims > mixer.rot_dim or mixer.rope_dims % 2:
@@ -144,7 +147,7 @@ def nibalix_spec_from_config(cfg: dict, name: str = "nibalix") -> HybridSpec:
                       width=int(cfg["width"]),
                       norm_eps=float(cfg["norm"]["eps"]),
                       residual_mult=float(cfg["residual_mult"]),
-                      conv_taps=int(cfg["canon"]["taps"]),
+                      conv_taps=int((cfg.get("canon") or {}).get("taps") or 0),
                       layers=tuple(layers))
 
 
@@ -169,10 +172,13 @@ def nibalix_config_from_spec(spec: HybridSpec) -> dict:
             fc = {"kind": "moe", "expert": {"ff": ls.mlp.ff},
                   "router": {"experts": ls.mlp.experts, "top": ls.mlp.top}}
         layers.append({"type": typ, "mixer": mc, "mlp": fc})
-    return {"architecture": "Nibalix", "canon": {"taps": spec.conv_taps},
-            "layers": layers, "norm": {"eps": spec.norm_eps},
-            "residual_mult": spec.residual_mult, "vocab": spec.vocab_size,
-            "width": spec.width}
+    out = {"architecture": "Nibalix", "layers": layers,
+           "norm": {"eps": spec.norm_eps},
+           "residual_mult": spec.residual_mult, "vocab": spec.vocab_size,
+           "width": spec.width}
+    if spec.conv_taps:
+        out["canon"] = {"taps": spec.conv_taps}
+    return out
 
 
 # ---------------------------------------------------------------- weights
@@ -195,7 +201,8 @@ class HybridLayer(nn.Module):
 
         f32 = torch.float32
         self.norm_w = P(D, dt=f32)
-        self.conv_w = P(D, spec.conv_taps, dt=f32)
+        if spec.conv_taps:      # 0: the mixer reads the normed input as it is
+            self.conv_w = P(D, spec.conv_taps, dt=f32)
         n_gate = 2 * D if ls.mlp is not None else D
         self.gate_w, self.gate_b = P(n_gate, D), P(n_gate, dt=f32)
         m = ls.mixer
@@ -256,7 +263,8 @@ class HybridLM(nn.Module):
         for i, (ls, L) in enumerate(zip(self.spec.layers, self.layers)):
             p = f"l{i}."
             out[p + "norm1"] = (L.norm_w, None)
-            out[p + "canon1"] = (L.conv_w, None)
+            if self.spec.conv_taps:
+                out[p + "canon1"] = (L.conv_w, None)
             out[p + "rg1"], out[p + "rg1.b"] = (L.gate_w, (0, D)), (L.gate_b, (0, D))
             m = ls.mixer
             if isinstance(m, LatentAttentionSpec):
@@ -344,7 +352,13 @@ def load_nibalix_checkpoint(path: str, dtype=torch.bfloat16, device=None) -> Hyb
     name = os.path.basename(os.path.normpath(path)) or "nibalix"
     model = HybridLM(nibalix_spec_from_config(cfg, name), dtype=dtype, device=device)
     tensors = load_file(os.path.join(path, "model.safetensors"))
-    model.load_tensors(tensors)
+    known = model._named_slices()
+    extra = sorted(k for k in tensors if k not in known)
+    if extra:
+        import sys
+        sys.stderr.write(f"[nibalix] ignoring {len(extra)} tensors the design "
+                         f"does not name: {extra[:4]}\n")
+    model.load_tensors({k: v for k, v in tensors.items() if k in known})
     return model
 
 

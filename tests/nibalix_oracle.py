@@ -133,7 +133,7 @@ def forward(cfg, W, tokens, dtype=F64, return_layers=False):
     for i, lc in enumerate(cfg["layers"]):
         p = f"l{i}."
         hs = [norm_offset(x, W[p + "norm1"], eps) for x in xs]
-        hm = canon(hs, W[p + "canon1"])
+        hm = canon(hs, W[p + "canon1"]) if cfg.get("canon") else hs
         mc = lc["mixer"]
         if lc["type"] == "latent_attention":
             src = mc.get("kv_from")
@@ -179,7 +179,8 @@ def random_weights(cfg, seed=0, scale=1.0):
     for i, lc in enumerate(cfg["layers"]):
         p, mc = f"l{i}.", lc["mixer"]
         W[p + "norm1"] = vec(D)
-        W[p + "canon1"] = (torch.randn(D, cfg["canon"]["taps"], generator=g) * 0.3).bfloat16().float()
+        if cfg.get("canon"):
+            W[p + "canon1"] = (torch.randn(D, cfg["canon"]["taps"], generator=g) * 0.3).bfloat16().float()
         W[p + "rg1"], W[p + "rg1.b"] = mat(D, D), vec(D, 0.5)
         if lc["type"] == "latent_attention":
             H, dn, rd, vd, r = mc["heads"], mc["dim"], mc["rot_dim"], mc["vdim"], mc["kv_rank"]

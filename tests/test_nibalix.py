@@ -557,6 +557,18 @@ def test_checkpoint_registry_and_trace_replay(tmp_path):
     assert rel_err(rd(2), la[8:9]) < 2e-4
 
 
+def test_optional_config_parts(dev):
+    """No input convolution, no window, default scale and rotation: what the
+    configuration leaves out is not computed (or takes the design's default)."""
+    cfg = mixed_cfg()
+    del cfg["canon"]
+    del cfg["layers"][0]["mixer"]["mask"]
+    cfg["layers"][3]["mixer"]["mask"] = None
+    W, eng = build(cfg, dev)
+    t = toks(17, cfg["vocab"], seed=80)
+    assert rel_err(run_portions(eng, t, [6, 1, 1, 9]), O.forward(cfg, W, t)) < tol(dev[1])
+
+
 def test_config_errors():
     cfg = mixed_cfg()
     bad = json.loads(json.dumps(cfg))
