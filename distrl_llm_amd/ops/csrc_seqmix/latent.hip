@@ -418,9 +418,10 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
 
 // ---- prompt tiles, all on MFMA: four waves share one tile of up to 16
 // queries of one head. Each 32-key block of the cache is staged in LDS once;
-// every wave forms the block's scores and fp32 softmax weights (the same in
-// all four), then takes every fourth 16-wide slice of the latent axis of the
-// weighted sum: O[q, f] += sum_k P[q, k] C[k, f] as MFMA with the weights
+// the waves share the block's score MFMAs (a 16-key tile and half of the
+// feature steps each, summed through LDS), every wave keeps the same fp32
+// softmax state, then takes every fourth 16-wide slice of the latent axis of
+// the weighted sum: O[q, f] += sum_k P[q, k] C[k, f] as MFMA with the weights
 // split into two bf16 terms (p = hi + lo, |p - hi - lo| <= 2^-17 p), so the
 // fp32 weights keep 16+ bits against the bf16 latents; accumulation is fp32.
 #define LC_NT 8      // latent slices per wave: kv_rank <= 4 * 8 * 16
@@ -446,7 +447,8 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
   const int lrow = l & 15, lk = l >> 4;
   bf16_t* q_lds = reinterpret_cast<bf16_t*>(smem);                 // [16][Wp]
   bf16_t* c_lds = q_lds + LT_TQ * Wp;                               // [32][Wp]
-  float* p_lds = reinterpret_cast<float*>(c_lds + LT_KB * Wp) + wave * (LT_TQ * LT_KB);
+  float* s_lds = reinterpret_cast<float*>(c_lds + LT_KB * Wp);     // [2][16][32] score halves
+  float* p_lds = s_lds + 2 * LT_TQ * LT_KB + wave * (LT_TQ * LT_KB);
 
   const int tile = blockIdx.x;
   const int hd = HEADS ? blockIdx.y * LT_TQ : blockIdx.y;
@@ -514,15 +516,31 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     __syncthreads();
     if (kb + 1 < kb_hi) key_rows(kb + 1);  // read again only after the next barrier
     const int j0 = lo + kb * LT_KB;
-    // scores of the 32 keys (two 16-key MFMA tiles), same in every wave
-    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    for (int ks = 0; ks < KS; ++ks) {
-      const int f0 = ks * 32 + lk * 8;
-      const bf16v8_t a = *reinterpret_cast<const bf16v8_t*>(q_lds + lrow * Wp + f0);
-      const bf16v8_t b0 = *reinterpret_cast<const bf16v8_t*>(c_lds + lrow * Wp + f0);
-      const bf16v8_t b1 = *reinterpret_cast<const bf16v8_t*>(c_lds + (16 + lrow) * Wp + f0);
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b0, s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, s1, 0, 0, 0);
+    // scores of the 32 keys: wave w forms the 16-key tile (w & 1) over one
+    // half (w >> 1) of the feature steps; the two halves are added through
+    // LDS and every wave then holds the whole 16 x 32 score block
+    {
+      const int u = wave & 1, hf = wave >> 1;
+      const int ksh = (KS + 1) / 2;
+      const int ks0 = hf * ksh, ks1 = min(KS, ks0 + ksh);
+      f32x4_t sp = {0.f, 0.f, 0.f, 0.f};
+      for (int ks = ks0; ks < ks1; ++ks) {
+        const int f0 = ks * 32 + lk * 8;
+        const bf16v8_t a = *reinterpret_cast<const bf16v8_t*>(q_lds + lrow * Wp + f0);
+        const bf16v8_t bk = *reinterpret_cast<const bf16v8_t*>(c_lds + (u * 16 + lrow) * Wp + f0);
+        sp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bk, sp, 0, 0, 0);
+      }
+      #pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        s_lds[(hf * LT_TQ + lk * 4 + rr) * LT_KB + u * 16 + lrow] = sp[rr];
+    }
+    __syncthreads();
+    f32x4_t s0, s1;
+    #pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int q = lk * 4 + rr;
+      s0[rr] = s_lds[q * LT_KB + lrow] + s_lds[(LT_TQ + q) * LT_KB + lrow];
+      s1[rr] = s_lds[q * LT_KB + 16 + lrow] + s_lds[(LT_TQ + q) * LT_KB + 16 + lrow];
     }
     float cr[4];
     #pragma unroll
@@ -718,8 +736,16 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     const bool heads = max_tile_queries == 1 && H > 1;
     if (!heads && max_tile_queries > 4) {
       // prompt portions: the four-wave all-MFMA kernel
-      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 4 * LT_TQ * LT_KB * 4;
-      if (ldsc <= 64 * 1024) {
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 6 * LT_TQ * LT_KB * 4;
+      if (ldsc <= 78 * 1024) {              // two workgroups per CU
+        static int raised = 0;
+        if ((int)ldsc > raised) {
+          TORCH_CHECK(hipFuncSetAttribute(
+                          reinterpret_cast<const void*>(latent_attention_coop_kernel<false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsc) == hipSuccess,
+                      "latent attention: cannot raise the LDS limit");
+          raised = (int)ldsc;
+        }
         latent_attention_coop_kernel<false><<<dim3(ntiles, H), 256, ldsc, stream>>>(
             reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
             reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
@@ -733,8 +759,16 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     if (heads) {
       // decoding: one token x up to 16 heads per workgroup, the key blocks
       // spread over blockIdx.z, merged by latent_combine
-      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 4 * LT_TQ * LT_KB * 4;
-      if (ldsc <= 64 * 1024) {
+      const size_t ldsc = (size_t)(LT_TQ + LT_KB) * LC_ROW(W) * 2 + 6 * LT_TQ * LT_KB * 4;
+      if (ldsc <= 78 * 1024) {
+        static int raised = 0;
+        if ((int)ldsc > raised) {
+          TORCH_CHECK(hipFuncSetAttribute(
+                          reinterpret_cast<const void*>(latent_attention_coop_kernel<true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsc) == hipSuccess,
+                      "latent attention: cannot raise the LDS limit");
+          raised = (int)ldsc;
+        }
         const int64_t groups = (int64_t)ntiles * SM_CDIV(H, LT_TQ);
         int ks = (int)std::min<int64_t>(32, std::max<int64_t>(1, 1024 / groups));
         if (window > 0) ks = (int)std::min<int64_t>(ks, SM_CDIV(window, LT_KB) + 1);
