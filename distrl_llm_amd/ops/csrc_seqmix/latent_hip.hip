@@ -2,7 +2,14 @@
 // Latent attention: cache write (latent RMS norm + rotated shared key part),
 // query rotation, and windowed softmax attention in latent space over the
 // paged cache. Prompt portions and single decode tokens run in the same
-// launch: one wave per (token, head).
+// step. Three attention kernels, chosen on the host:
+//   latent_attention_coop    bf16 default: four waves per tile of <= 16 rows
+//                            (queries of one head, or heads of one decoded
+//                            token), key blocks staged in LDS, scores and
+//                            weighted sum on MFMA
+//   latent_attention_tiled   bf16 fallback (tile too wide for LDS, tiny
+//                            portions): MFMA scores, fp32 FMA weighted sum
+//   latent_attention         one wave per (token, head): fp32 models, any size
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 #include "seqmix_common.h"
