@@ -9,10 +9,11 @@ the prompt's pages and state), with the same call signature as the dense
 :class:`Engine`, so the batcher, the server and the command line drive
 either. A trace replay (``bin/trace_run``) calls the same step directly.
 
-Numerics: the residual stream, norms, convolution, rotary angles,
-attention scores/softmax, recurrent state, router and the gated residual
-sum are fp32; matrix products run in the model dtype with fp32
-accumulation (true fp32 when the model dtype is fp32).
+Numerics: the residual stream, norms, the block's convolution, rotary
+angles, attention scores and weights, recurrent state with its decays,
+gates and unit norms, router and the residual sum are fp32; matrix
+products run in the model dtype with fp32 accumulation (true fp32 when the
+model dtype is fp32).
 """
 
 from __future__ import annotations
@@ -23,7 +24,8 @@ import torch
 import torch.nn.functional as F
 
 from ..config import EngineConfig, SamplingParams
-from ..models.hybrid import HybridLM, LatentAttentionSpec
+from ..models.hybrid import (DeltaRuleSpec, GluSpec, HybridLM,
+                             LatentAttentionSpec, SinkAttentionSpec)
 from ..ops import functional as OF
 from ..ops import seqmix as SM
 from ..utils.trace import trace_range
@@ -297,51 +299,131 @@ class HybridEngine:
             q.context_len += len(toks)
         return logits
 
+    # ---- mixers: (layer index, specs, weights, mixer input) -> [T, width]
+
+    def _mix_latent(self, i, m, L, hm, meta):
+        S, dt, T = self.spec, self.dtype, hm.shape[0]
+        own = m.kv_from is None
+        proj = F.linear(hm, L.in_w)
+        cache = self.pool.layer_rows(S, i)
+        q_rot = SM.latent_prepare(
+            proj, m.heads, m.dim, m.rot_dim, m.kv_rank, own,
+            L.latent_norm_w if own else None, S.norm_eps, meta["positions"],
+            m.rope_base, m.rope_dims, meta["page_slot"], cache)
+        q_nope = proj[:, :m.q_size].view(T, m.heads, m.dim + m.rot_dim)
+        q_lat = torch.bmm(q_nope[..., :m.dim].transpose(0, 1), L.uk)
+        o_lat = SM.latent_window_attention(
+            q_lat, q_rot, cache, m.kv_rank, meta["block_tables"],
+            self.pool.block_size, meta["cu"], meta["tok_seq"],
+            meta["positions"], m.window, m.scale, dt,
+            tiles=meta["tiles"], max_tile=meta["max_tile"])
+        v = torch.bmm(o_lat, L.uv.transpose(1, 2))
+        return F.linear(v.transpose(0, 1).reshape(T, m.heads * m.vdim), L.out_w)
+
+    def _mix_mingru(self, i, m, L, hm, meta):
+        zxg = F.linear(hm, L.in_w)
+        a = SM.mingru_scan(zxg, L.in_b, self.slots.recurrent[i], meta["cu"],
+                           meta["slots"], self.dtype, meta["scan_chunks"],
+                           meta["scan_cu"])
+        return F.linear(a, L.out_w)
+
+    def _mix_sink_attention(self, i, m, L, hm, meta, shared):
+        """``shared`` carries the first value-mixing layer's fresh values of
+        this step's tokens to the later mixing layers."""
+        proj = F.linear(hm, L.in_w)
+        cache = self.pool.layer_rows(self.spec, i)
+        v_first = shared.get(("v", m.v_first)) if m.v_first is not None else None
+        q = SM.rope_kv_write(proj, m.heads, m.kv_heads, m.dim, m.vdim,
+                             meta["positions"], m.rope_base, m.rope_dims,
+                             meta["page_slot"], cache, L.vmix, v_first)
+        if m.v_mix and m.v_first is None:
+            shared[("v", i)] = proj[:, m.q_size + m.k_size:]
+        o = SM.sink_attention(q, cache, m.heads, m.kv_heads, m.dim, m.vdim,
+                              meta["block_tables"], self.pool.block_size,
+                              meta["cu"], meta["tok_seq"], meta["positions"],
+                              m.scale, m.softcap, L.sink, L.talk, self.dtype,
+                              tiles=meta["tiles"], max_tile=meta["max_tile"])
+        return F.linear(o, L.out_w)
+
+    def _mix_delta(self, i, m, L, hm, meta):
+        proj = F.linear(hm, L.in_w)
+        C = m.conv_channels
+        qkv = SM.tap_conv_silu(proj[:, :C], L.conv_w, self.slots.mixer_tails[i],
+                               meta["cu"], meta["tok_seq"], meta["slots"],
+                               self.dtype)
+        ab = F.linear(hm.float(), L.ab_w)            # fp32 decay / strength inputs
+        o = SM.gated_delta_rule(qkv, proj[:, C:], ab, L.a_log, L.dt_bias,
+                                L.onorm_w, self.spec.norm_eps,
+                                self.slots.recurrent[i], meta["cu"],
+                                meta["slots"], m.heads, m.kv_heads, m.dim,
+                                m.vdim, self.dtype)
+        return F.linear(o, L.out_w)
+
+    def _mixer(self, i, ls, L, hm, meta, shared):
+        m = ls.mixer
+        if isinstance(m, LatentAttentionSpec):
+            return self._mix_latent(i, m, L, hm, meta)
+        if isinstance(m, SinkAttentionSpec):
+            return self._mix_sink_attention(i, m, L, hm, meta, shared)
+        if isinstance(m, DeltaRuleSpec):
+            return self._mix_delta(i, m, L, hm, meta)
+        return self._mix_mingru(i, m, L, hm, meta)
+
+    # ---- feed-forwards: -> (main output, second addend or None)
+
+    def _ff(self, f, L, hb):
+        if isinstance(f, GluSpec):
+            return F.linear(SM.capped_glu(F.linear(hb, L.gu_w), f.limit),
+                            L.down_w), None
+        if f.routing == "all":
+            idx, wts = SM.moe_route_all(hb, L.router_w, L.correction, f.top,
+                                        f.scale)
+            y = SM.moe_experts_glu(hb, idx, wts, L.exp_gu, L.exp_down, f.limit)
+            if f.shared is None:
+                return y, None
+            return y, F.linear(SM.capped_glu(F.linear(hb, L.shared_gu),
+                                             f.shared.limit), L.shared_down)
+        idx, wts = SM.moe_route(hb, L.router_w, L.router_b, f.top)
+        return SM.moe_experts(hb, idx, wts, L.exp_gu, L.exp_down), None
+
+    # ---- block arrangements
+
     def _forward(self, tokens, meta, want_rows, capture=None) -> torch.Tensor:
         S, M, dt = self.spec, self.model, self.dtype
-        eps, mult = S.norm_eps, S.residual_mult
-        T = tokens.shape[0]
-        pos, cu, slots = meta["positions"], meta["cu"], meta["slots"]
-        bs = self.pool.block_size
+        if S.block == "sandwich":
+            x = self._layers_sandwich(tokens, meta, capture)
+        else:
+            x = self._layers_parallel_gated(tokens, meta, capture)
+        if want_rows.numel() == 0:
+            return torch.empty(0, S.vocab_size, dtype=torch.float32,
+                               device=x.device)
+        _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, S.norm_eps, dt)
+        return F.linear(hb, M.head).float()
 
+    def _layers_parallel_gated(self, tokens, meta, capture):
+        """One norm per layer feeds the mixer (through the block's short
+        convolution) and the feed-forward; their outputs enter the residual
+        through sigmoid gates."""
+        S, M, dt = self.spec, self.model, self.dtype
+        eps, mult = S.norm_eps, S.residual_mult
+        shared = {}
         x, _ = SM.offset_rmsnorm(M.embed[tokens], M.embed_norm_w, eps, dt)
         h32, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt)
         last = S.num_layers - 1
         for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
             if S.conv_taps:
-                hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i], cu,
-                                        meta["tok_seq"], slots, dt)
+                hm = SM.causal_tap_conv(h32, L.conv_w, self.slots.tails[i],
+                                        meta["cu"], meta["tok_seq"],
+                                        meta["slots"], dt)
             else:
                 hm = hb
             gates = F.linear(hb, L.gate_w)
-            m = ls.mixer
-            if isinstance(m, LatentAttentionSpec):
-                own = m.kv_from is None
-                proj = F.linear(hm, L.in_w)
-                cache = self.pool.layer_rows(S, i)
-                q_rot = SM.latent_prepare(
-                    proj, m.heads, m.dim, m.rot_dim, m.kv_rank, own,
-                    L.latent_norm_w if own else None, eps, pos, m.rope_base,
-                    m.rope_dims, meta["page_slot"], cache)
-                q_nope = proj[:, :m.q_size].view(T, m.heads, m.dim + m.rot_dim)
-                q_lat = torch.bmm(q_nope[..., :m.dim].transpose(0, 1), L.uk)
-                o_lat = SM.latent_window_attention(
-                    q_lat, q_rot, cache, m.kv_rank, meta["block_tables"], bs,
-                    cu, meta["tok_seq"], pos, m.window, m.scale, dt,
-                    tiles=meta["tiles"], max_tile=meta["max_tile"])
-                v = torch.bmm(o_lat, L.uv.transpose(1, 2))
-                y = F.linear(v.transpose(0, 1).reshape(T, m.heads * m.vdim),
-                             L.out_w)
-            else:
-                zxg = F.linear(hm, L.in_w)
-                a = SM.mingru_scan(zxg, L.in_b, self.slots.recurrent[i], cu,
-                                   slots, dt, meta["scan_chunks"],
-                                   meta["scan_cu"])
-                y = F.linear(a, L.out_w)
+            y = self._mixer(i, ls, L, hm, meta, shared)
             f = None
             if ls.mlp is not None:
-                idx, wts = SM.moe_route(hb, L.router_w, L.router_b, ls.mlp.top)
-                f = SM.moe_experts(hb, idx, wts, L.exp_gu, L.exp_down)
+                f, f2 = self._ff(ls.mlp, L, hb)
+                if f2 is not None:
+                    f = f.float() + f2.float()
             if i < last:
                 h32, hb = SM.gated_residual_norm(
                     x, y, f, gates, L.gate_b, mult, M.layers[i + 1].norm_w,
@@ -350,11 +432,33 @@ class HybridEngine:
                 SM.gated_residual_add(x, y, f, gates, L.gate_b, mult)
             if capture is not None:
                 capture.append(x.clone())
-        if want_rows.numel() == 0:
-            return torch.empty(0, S.vocab_size, dtype=torch.float32,
-                               device=x.device)
-        _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, eps, dt)
-        return F.linear(hb, M.head).float()
+        return x
+
+    def _layers_sandwich(self, tokens, meta, capture):
+        """x += post(mixer(pre(x))), then x += post(ff(pre(x))): every
+        sublayer has an offset RMS norm before and after it. The residual
+        update, the sublayer's closing norm and the next opening norm are
+        one kernel."""
+        S, M, dt = self.spec, self.model, self.dtype
+        eps = S.norm_eps
+        shared = {}
+        x = M.embed[tokens].float()
+        _, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt)
+        last = S.num_layers - 1
+        for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
+            y = self._mixer(i, ls, L, hb, meta, shared)
+            nxt = M.layers[i + 1].norm_w if i < last else None
+            r = SM.sandwich_residual_norm(
+                x, y, None, L.post_w,
+                L.ff_norm_w if ls.mlp is not None else nxt, eps, dt)
+            if ls.mlp is not None:
+                f, f2 = self._ff(ls.mlp, L, r[1])
+                r = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, nxt, eps, dt)
+            if r is not None:
+                hb = r[1]
+            if capture is not None:
+                capture.append(x.clone())
+        return x
 
     def score(self, ids: Seq[int]) -> torch.Tensor:
         """Teacher-forced logits of every position of one token sequence

@@ -3,15 +3,18 @@
 Two pools, both handed out and taken back by the engine as sequences
 come and go:
 
-* :class:`LatentCachePool` — paged rows ``[latent | rotated key part]``
-  for every attention layer that owns a cache (layers that read another
-  layer's cache own none). Block ids come from the same refcounting
-  :class:`BlockAllocator` as the dense models' K/V pool, so a forked
-  candidate shares its prompt's full pages.
+* :class:`LatentCachePool` — paged rows for every attention layer that owns
+  a cache: ``[latent | rotated key part]`` for latent attention (layers
+  that read another layer's cache own none), ``[keys of all kv heads |
+  values of all kv heads]`` for grouped-query attention. Block ids come
+  from the same refcounting :class:`BlockAllocator` as the dense models'
+  K/V pool, so a forked candidate shares its prompt's full pages.
 * :class:`StateSlotPool` — fixed-size fp32 state per live sequence: the
-  last ``taps - 1`` inputs of every layer's short convolution and the
-  state vector of every recurrent layer. A slot is zeroed when it is
-  handed out, so whatever its previous owner left cannot leak.
+  last ``taps - 1`` inputs of every short convolution (the block's own, or
+  a delta-rule layer's over its q/k/v channels) and the state of every
+  recurrent layer (a vector for minGRU, a matrix per head for the delta
+  rule). A slot is zeroed when it is handed out, so whatever its previous
+  owner left cannot leak.
 """
 
 from __future__ import annotations
@@ -20,7 +23,8 @@ from typing import Dict, List
 
 import torch
 
-from ..models.hybrid import HybridSpec, LatentAttentionSpec, MinGRUSpec
+from ..models.hybrid import (DeltaRuleSpec, HybridSpec, LatentAttentionSpec,
+                             MinGRUSpec, SinkAttentionSpec)
 from .kvcache import BlockAllocator
 
 
@@ -37,13 +41,19 @@ class LatentCachePool:
         self.rows: Dict[int, torch.Tensor] = {}
         for i, ls in enumerate(spec.layers):
             m = ls.mixer
-            if isinstance(m, LatentAttentionSpec) and m.kv_from is None:
+            if self._owns_rows(m):
                 self.rows[i] = torch.zeros((num_blocks + 1) * block_size, m.cache_width,
                                            dtype=dtype, device=device)
 
+    @staticmethod
+    def _owns_rows(m) -> bool:
+        return (isinstance(m, SinkAttentionSpec)
+                or (isinstance(m, LatentAttentionSpec) and m.kv_from is None))
+
     def layer_rows(self, spec: HybridSpec, layer: int) -> torch.Tensor:
         m = spec.layers[layer].mixer
-        return self.rows[layer if m.kv_from is None else m.kv_from]
+        src = getattr(m, "kv_from", None)
+        return self.rows[layer if src is None else src]
 
     @staticmethod
     def blocks_for(num_tokens: int, block_size: int) -> int:
@@ -52,8 +62,7 @@ class LatentCachePool:
     @staticmethod
     def bytes_per_block(spec: HybridSpec, block_size: int, dtype) -> int:
         w = sum(ls.mixer.cache_width for ls in spec.layers
-                if isinstance(ls.mixer, LatentAttentionSpec)
-                and ls.mixer.kv_from is None)
+                if LatentCachePool._owns_rows(ls.mixer))
         return max(1, w) * block_size * torch.tensor([], dtype=dtype).element_size()
 
     def copy_block(self, src: int, dst: int) -> None:
@@ -71,12 +80,19 @@ class StateSlotPool:
         self.tails: List[torch.Tensor] = [
             torch.zeros(num_slots + 1, k, D, dtype=torch.float32, device=device)
             for _ in spec.layers]
-        # recurrent state: layer index -> [slots + 1, width] fp32
+        # recurrent state: layer index -> [slots + 1, state size] fp32
         self.recurrent: Dict[int, torch.Tensor] = {
-            i: torch.zeros(num_slots + 1, ls.mixer.width, dtype=torch.float32,
+            i: torch.zeros(num_slots + 1, ls.mixer.state_size, dtype=torch.float32,
                            device=device)
             for i, ls in enumerate(spec.layers)
-            if isinstance(ls.mixer, MinGRUSpec)}
+            if isinstance(ls.mixer, (MinGRUSpec, DeltaRuleSpec))}
+        # a mixer's own short convolution: layer index ->
+        # [slots + 1, taps - 1, channels] fp32
+        self.mixer_tails: Dict[int, torch.Tensor] = {
+            i: torch.zeros(num_slots + 1, ls.mixer.taps - 1, ls.mixer.conv_channels,
+                           dtype=torch.float32, device=device)
+            for i, ls in enumerate(spec.layers)
+            if isinstance(ls.mixer, DeltaRuleSpec)}
         self._free = list(range(num_slots - 1, -1, -1))
 
     @property
@@ -84,7 +100,8 @@ class StateSlotPool:
         return len(self._free)
 
     def _tensors(self):
-        return list(self.tails) + list(self.recurrent.values())
+        return (list(self.tails) + list(self.recurrent.values())
+                + list(self.mixer_tails.values()))
 
     def alloc(self) -> int:
         if not self._free:

@@ -147,3 +147,81 @@ def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
             x, mix, ff, gates, gate_b, mult, next_w, eps, _bf16(out_dtype))
     R.gated_residual_add(x, mix, ff, gates, gate_b, mult)
     return R.offset_rmsnorm(x, next_w, eps, out_dtype)
+
+
+# ------------------------------------------------- sandwich-block mechanisms
+
+def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
+    """Fused sublayer tail: x += rms_unit(y [+ y2]) * (1 + post_w) on the
+    fp32 residual (in place), then, with ``next_w``, the next offset RMS
+    norm of the new residual -> (fp32, out_dtype); None without."""
+    if x.is_cuda:
+        r = _ext("sandwich_residual_norm").sandwich_residual_norm(
+            x, y.contiguous(), None if y2 is None else y2.contiguous(), post_w,
+            next_w, eps, _bf16(out_dtype))
+        return None if next_w is None else r
+    return R.sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype)
+
+
+def rope_kv_write(proj, heads, kv_heads, dim, vdim, positions, rope_base,
+                  rope_dims, page_slot, cache, vmix=None, v_first=None):
+    if proj.is_cuda:
+        return _ext("rope_kv_write").rope_kv_write(
+            proj, heads, kv_heads, dim, vdim, positions, rope_base, rope_dims,
+            page_slot, cache, vmix, v_first)
+    return R.rope_kv_write(proj, heads, kv_heads, dim, vdim, positions,
+                           rope_base, rope_dims, page_slot, cache, vmix, v_first)
+
+
+def sink_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
+                   block_size, cu, tok_seq, positions, scale, softcap, sink,
+                   talk, out_dtype, tiles=None, max_tile=0):
+    """``tiles`` (from :func:`query_tiles`) selects the tiled MFMA kernel
+    for bf16 prompt portions; decode steps and fp32 models run one wave per
+    (token, head)."""
+    if q.is_cuda:
+        return _ext("sink_attention").sink_attention(
+            q, cache, heads, kv_heads, dim, vdim, block_tables, block_size,
+            tok_seq, positions, scale, softcap, sink, talk, tiles, max_tile)
+    return R.sink_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
+                            block_size, cu, positions, scale, softcap, sink,
+                            talk, out_dtype)
+
+
+def tap_conv_silu(x, w, tails, cu, tok_seq, slots, out_dtype):
+    """``x`` may be a column slice of a wider row-major matrix."""
+    if x.is_cuda:
+        return _ext("tap_conv_silu").tap_conv_silu(x, w, tails, cu, tok_seq,
+                                                   slots, _bf16(out_dtype))
+    return R.tap_conv_silu(x, w, tails, cu, slots, out_dtype)
+
+
+def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
+                     slots, heads, kv_heads, dim, vdim, out_dtype):
+    if qkv.is_cuda:
+        return _ext("gated_delta_rule").gated_delta_rule(
+            qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu, slots,
+            heads, kv_heads, dim, vdim)
+    return R.gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps,
+                              state, cu, slots, heads, kv_heads, dim, vdim,
+                              out_dtype)
+
+
+def capped_glu(gu, limit):
+    if gu.is_cuda:
+        return _ext("capped_glu").capped_glu(gu, limit)
+    return R.capped_glu(gu, limit)
+
+
+def moe_route_all(h, router_w, correction, top, scale):
+    if h.is_cuda:
+        return _ext("moe_route_all").moe_route_all(h, router_w, correction,
+                                                   top, scale)
+    return R.moe_route_all(h, router_w, correction, top, scale)
+
+
+def moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit):
+    if h.is_cuda:
+        return _ext("moe_experts_glu").moe_experts_glu(h, idx, wts, exp_gu,
+                                                       exp_down, limit)
+    return R.moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit)

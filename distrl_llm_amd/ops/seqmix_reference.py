@@ -180,3 +180,192 @@ def gated_residual_add(x, mix, ff, gates, gate_b, mult):
         acc = acc + ff.float() * g[:, D:2 * D]
     x.add_(acc, alpha=mult)
     return x
+
+
+# ------------------------------------------------- sandwich-block mechanisms
+
+def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
+    """x += rms_unit(y [+ y2]) * (1 + post_w) on the fp32 residual, in
+    place; with ``next_w`` also returns the next offset RMS norm of the new
+    residual as (fp32, out_dtype), else None."""
+    s = y.float() if y2 is None else y.float() + y2.float()
+    x.add_(s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps)
+           * (1.0 + post_w.float()))
+    if next_w is None:
+        return None
+    return offset_rmsnorm(x, next_w, eps, out_dtype)
+
+
+def _rotate_pairs(v, positions, base, dims):
+    """Rotate entries (2i, 2i+1) of the first ``dims`` of the last axis by
+    position * base^(-2i/dims) (fp32 in/out). v [T, heads, n]."""
+    if dims == 0:
+        return v
+    half = dims // 2
+    i = torch.arange(half, device=v.device, dtype=torch.float32)
+    freq = torch.exp2(i * (-2.0 / dims) * torch.log2(
+        torch.tensor(float(base), device=v.device)))
+    ang = positions.to(torch.float32)[:, None] * freq[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    rot = torch.stack([a * c - b * s, b * c + a * s], -1).flatten(-2)
+    return torch.cat([rot, v[..., dims:]], -1)
+
+
+def rope_kv_write(proj, heads, kv_heads, dim, vdim, positions, rope_base,
+                  rope_dims, page_slot, cache, vmix, v_first):
+    """From packed [q | k | v] projection rows: rotate q and k, blend v with
+    ``v_first`` ((1 - vmix) v + vmix v_first, when given) and write
+    [k | v] into ``cache`` rows ``page_slot``. Returns the rotated queries
+    [T, heads, dim] in the projection's dtype."""
+    T = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q = _rotate_pairs(proj[:, :nq].float().view(T, heads, dim), positions,
+                      rope_base, rope_dims)
+    k = _rotate_pairs(proj[:, nq:nq + nk].float().view(T, kv_heads, dim),
+                      positions, rope_base, rope_dims)
+    v = proj[:, nq + nk:].float()
+    if v_first is not None:
+        lam = vmix.float().reshape(())
+        v = (1.0 - lam) * v + lam * v_first.float()
+    cache[page_slot.long()] = torch.cat([k.reshape(T, nk), v], -1).to(cache.dtype)
+    return q.to(proj.dtype)
+
+
+def sink_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
+                   block_size, cu, positions, scale, softcap, sink, talk,
+                   out_dtype):
+    """Causal grouped-query softmax attention over paged [k | v] rows.
+
+    score = q.k * scale, then softcap * tanh(score / softcap) when softcap
+    > 0; the softmax denominator also holds exp(sink[h]) (sink None: plain
+    softmax); the heads' weights are mixed by ``talk`` [H, H]
+    (w_h <- sum_g talk[h, g] w_g) before head h reads the values of its own
+    kv head. q [T, H, dim] -> [T, H * vdim]."""
+    T = q.shape[0]
+    rep = heads // kv_heads
+    nk = kv_heads * dim
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32, device=q.device)
+    cu_l, pos_l = cu.tolist(), positions.tolist()
+    for b in range(len(cu_l) - 1):
+        a, e = cu_l[b], cu_l[b + 1]
+        if e == a:
+            continue
+        j = torch.arange(0, pos_l[e - 1] + 1, device=cache.device)
+        rows = block_tables[b].long()[j // block_size] * block_size + j % block_size
+        kv = cache[rows].float()
+        k = kv[:, :nk].view(-1, kv_heads, dim).repeat_interleave(rep, 1)
+        v = kv[:, nk:].view(-1, kv_heads, vdim).repeat_interleave(rep, 1)
+        s = torch.einsum("thd,jhd->htj", q[a:e].float(), k) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        ok = j[None, :] <= positions[a:e].long()[:, None]
+        s = s.masked_fill(~ok[None], float("-inf"))
+        if sink is not None:
+            s = torch.cat([s, sink.float()[:, None, None].expand(-1, e - a, 1)], -1)
+        w = torch.softmax(s, -1)[..., :j.numel()]
+        if talk is not None:
+            w = torch.einsum("hg,gtj->htj", talk.float(), w)
+        out[a:e] = torch.einsum("htj,jhd->thd", w, v)
+    return out.reshape(T, heads * vdim).to(out_dtype)
+
+
+def tap_conv_silu(x, w, tails, cu, slots, out_dtype):
+    """silu(sum_j w[:, j] * x_(t - taps + 1 + j)) per channel and sequence;
+    inputs before the portion come from ``tails[slot]`` (fp32
+    [slots, taps-1, C]), which is advanced to the portion's end."""
+    taps = w.shape[1]
+    x = x.float()
+    out = torch.empty_like(x)
+    cu_l, slots_l = cu.tolist(), slots.tolist()
+    for b, s in enumerate(slots_l):
+        a, e = cu_l[b], cu_l[b + 1]
+        if e == a:
+            continue
+        ext = torch.cat([tails[s], x[a:e]], 0)
+        n = e - a
+        acc = torch.zeros_like(x[a:e])
+        for j in range(taps):
+            acc += w[:, j] * ext[j:j + n]
+        out[a:e] = acc * torch.sigmoid(acc)
+        if taps > 1:
+            tails[s] = ext[ext.shape[0] - (taps - 1):]
+    return out.to(out_dtype)
+
+
+def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
+                     slots, heads, kv_heads, dim, vdim, out_dtype):
+    """Gated delta rule over a flat batch.
+
+    qkv [T, 2 G dim + H vdim] (after convolution and SiLU), gate [T, H vdim]
+    pre-activation, ab fp32 [T, 2H] = [write strength | step] pre-activations.
+    Per head: q, k -> unit vectors (q also / sqrt(dim));
+    beta = sigmoid(b); decay = exp(-exp(a_log) softplus(a + dt_bias));
+    S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
+    out = o / rms(o) * onorm_w * silu(gate). state fp32
+    [slots, H * dim * vdim], advanced in place."""
+    T = qkv.shape[0]
+    H, G = heads, kv_heads
+    rep = H // G
+    n = G * dim
+    x = qkv.float()
+    q = x[:, :n].view(T, G, dim)
+    k = x[:, n:2 * n].view(T, G, dim)
+    v = x[:, 2 * n:].view(T, H, vdim)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(ab[:, :H].float())
+    decay = torch.exp(-torch.exp(a_log.float())
+                      * F.softplus(ab[:, H:].float() + dt_bias.float()))
+    o = torch.empty(T, H, vdim, dtype=torch.float32, device=qkv.device)
+    cu_l, slots_l = cu.tolist(), slots.tolist()
+    for b, s in enumerate(slots_l):
+        S = state[s].view(H, dim, vdim).clone()
+        for t in range(cu_l[b], cu_l[b + 1]):
+            S = decay[t][:, None, None] * S
+            u = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
+            S = S + k[t][:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hkv,hk->hv", S, q[t])
+        state[s] = S.reshape(-1)
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * onorm_w.float()
+    g = gate.float().view(T, H, vdim)
+    return (o * g * torch.sigmoid(g)).reshape(T, H * vdim).to(out_dtype)
+
+
+def capped_glu(gu, limit):
+    """gu [T, 2ff] = [gate | up]: g = min(gate, limit), u = clamp(up,
+    +-limit); g * sigmoid(1.702 g) * (u + 1), in gu's dtype."""
+    ff = gu.shape[1] // 2
+    g = gu[:, :ff].float().clamp(max=limit)
+    u = gu[:, ff:].float().clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(gu.dtype)
+
+
+def moe_route_all(h, router_w, correction, top, scale):
+    """fp32 router over every output: s = softmax(W h); the ``top`` largest
+    s + correction are chosen (ties: lowest index first); weights =
+    s[chosen] * scale, not renormalised."""
+    s = torch.softmax(F.linear(h.float(), router_w.float()), -1)
+    c = s if correction is None else s + correction.float()
+    _, idx = torch.sort(c, dim=-1, descending=True, stable=True)
+    idx = idx[:, :top]
+    return idx.to(torch.int32), torch.gather(s, 1, idx) * scale
+
+
+def moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit):
+    """Mixture of clamped-GLU experts; indices >= the number of expert
+    weight sets name identity experts whose output is the input itself."""
+    T, D = h.shape
+    E = exp_gu.shape[0]
+    out = torch.zeros(T, D, dtype=torch.float32, device=h.device)
+    for e in range(E):
+        hit = idx == e
+        rows = hit.any(-1).nonzero().flatten()
+        if rows.numel() == 0:
+            continue
+        act = capped_glu(F.linear(h[rows], exp_gu[e]), limit)
+        y = F.linear(act, exp_down[e]).float()
+        out[rows] += (wts[rows] * hit[rows]).sum(-1, keepdim=True) * y
+    ident = (wts * (idx >= E)).sum(-1, keepdim=True)
+    return out + ident * h.float()
