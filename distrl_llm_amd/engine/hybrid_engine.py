@@ -448,14 +448,12 @@ class HybridEngine:
         for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
             y = self._mixer(i, ls, L, hb, meta, shared)
             nxt = M.layers[i + 1].norm_w if i < last else None
-            r = SM.sandwich_residual_norm(
+            hb = SM.sandwich_residual_norm(
                 x, y, None, L.post_w,
                 L.ff_norm_w if ls.mlp is not None else nxt, eps, dt)
             if ls.mlp is not None:
-                f, f2 = self._ff(ls.mlp, L, r[1])
-                r = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, nxt, eps, dt)
-            if r is not None:
-                hb = r[1]
+                f, f2 = self._ff(ls.mlp, L, hb)
+                hb = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, nxt, eps, dt)
             if capture is not None:
                 capture.append(x.clone())
         return x

@@ -36,6 +36,36 @@ std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
 torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
                           torch::Tensor exp_gu, torch::Tensor exp_down);
 
+std::vector<torch::Tensor> moe_route_all(torch::Tensor h, torch::Tensor router_w,
+                                         c10::optional<torch::Tensor> correction,
+                                         int64_t top, double scale);
+torch::Tensor moe_experts_glu(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                              torch::Tensor exp_gu, torch::Tensor exp_down, double limit);
+torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tails,
+                            torch::Tensor cu, torch::Tensor tok_seq, torch::Tensor slots,
+                            bool out_bf16);
+c10::optional<torch::Tensor> sandwich_residual_norm(
+    torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2, torch::Tensor post_w,
+    c10::optional<torch::Tensor> next_w, double eps, bool out_bf16);
+torch::Tensor capped_glu(torch::Tensor gu, double limit);
+torch::Tensor rope_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
+                            int64_t vdim, torch::Tensor positions, double rope_base,
+                            int64_t rope_dims, torch::Tensor page_slot, torch::Tensor cache,
+                            c10::optional<torch::Tensor> vmix,
+                            c10::optional<torch::Tensor> v_first);
+torch::Tensor sink_attention(torch::Tensor q, torch::Tensor cache, int64_t heads,
+                             int64_t kv_heads, int64_t dim, int64_t vdim,
+                             torch::Tensor block_tables, int64_t block_size,
+                             torch::Tensor tok_seq, torch::Tensor positions, double scale,
+                             double softcap, c10::optional<torch::Tensor> sink,
+                             c10::optional<torch::Tensor> talk,
+                             c10::optional<torch::Tensor> tiles, int64_t max_tile_queries);
+torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Tensor ab,
+                               torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
+                               double eps, torch::Tensor state, torch::Tensor cu,
+                               torch::Tensor slots, int64_t heads, int64_t kv_heads,
+                               int64_t dim, int64_t vdim);
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("offset_rmsnorm", &offset_rmsnorm, "offset-weight RMS norm -> (fp32, dtype)");
   m.def("gated_residual_add", &gated_residual_add, "gated parallel-residual update");
@@ -48,4 +78,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("mingru_scan", &mingru_scan, "minGRU scan with per-slot fp32 state");
   m.def("moe_route", &moe_route, "fp32 top-k router");
   m.def("moe_experts", &moe_experts, "grouped-GEMM mixture of SiLU-gated experts");
+  m.def("moe_route_all", &moe_route_all, "fp32 router: softmax over all, corrected choice");
+  m.def("moe_experts_glu", &moe_experts_glu,
+        "grouped-GEMM mixture of clamped-GLU experts with identity experts");
+  m.def("tap_conv_silu", &tap_conv_silu, "short causal conv + SiLU with slot tails");
+  m.def("sandwich_residual_norm", &sandwich_residual_norm,
+        "closing norm + residual sum + next opening norm");
+  m.def("capped_glu", &capped_glu, "clamped GLU activation");
+  m.def("rope_kv_write", &rope_kv_write, "pair rotary on q/k, value blend, K/V cache write");
+  m.def("sink_attention", &sink_attention,
+        "paged GQA with capped scores, sinks and head mixing");
+  m.def("gated_delta_rule", &gated_delta_rule, "gated delta rule with per-slot fp32 state");
 }

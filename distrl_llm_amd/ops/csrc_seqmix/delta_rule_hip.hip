@@ -1,0 +1,222 @@
+#include "hip/hip_runtime.h"
+// Gated delta rule over a flat varlen batch, fp32 matrix state per (slot,
+// head). Three kernels:
+//   delta_prepare   per token: q, k of every q/k head made unit vectors (q
+//                   also / sqrt(dim)), write strength beta = sigmoid(b) and
+//                   decay = exp(-exp(a_log) softplus(a + dt_bias)), all fp32
+//   delta_scan      per (sequence row, head, block of value columns): walks
+//                   the row's tokens in order with the state in registers,
+//                   S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
+//   delta_finish    per (token, head): o / rms(o) * norm_w * silu(gate)
+// The scan is strictly sequential over a row's tokens, so a prompt cut into
+// portions gives bit-identical states and outputs.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include "seqmix_common.h"
+
+namespace {
+
+#define DR_ROWS 32    // state rows (key dims) held by one lane
+
+// qkv row = [q (G dk) | k (G dk) | v (H vd)] after convolution and SiLU.
+// One workgroup per token; wave w normalises q/k heads w, w + 4, ...
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    const T* __restrict__ qkv, int C, const float* __restrict__ ab,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, int H, int G,
+    int dk, int dkp, float* __restrict__ qn, float* __restrict__ kn,
+    float* __restrict__ beta, float* __restrict__ decay) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* row = qkv + t * C;
+  for (int job = wave; job < 2 * G; job += 4) {
+    const bool is_k = job >= G;
+    const int g = is_k ? job - G : job;
+    const T* src = row + (is_k ? G * dk : 0) + g * dk;
+    float ss = 0.f;
+    for (int k = lane; k < dk; k += 64) {
+      const float v = to_f(src[k]);
+      ss += v * v;
+    }
+    ss = sm_wave_sum(ss);
+    float inv = 1.0f / sqrtf(ss + 1e-6f);
+    if (!is_k) inv *= 1.0f / sqrtf((float)dk);
+    float* dst = (is_k ? kn : qn) + (t * G + g) * dkp;
+    for (int k = lane; k < dkp; k += 64) dst[k] = (k < dk) ? to_f(src[k]) * inv : 0.f;
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    beta[t * H + h] = sm_sigmoid(ab[t * 2 * H + h]);
+    const float z = ab[t * 2 * H + H + h] + dt_bias[h];
+    const float sp = (z > 20.f) ? z : log1pf(expf(z));
+    decay[t * H + h] = expf(-expf(a_log[h]) * sp);
+  }
+}
+
+// One wave per (row, head, 64 / KS value columns). Lane = (column, ks): it
+// holds rows ks * 32 .. ks * 32 + 31 of its column; dot products over the key
+// axis are finished with shuffles over the KS lanes of a column.
+template <typename T, int KS>
+__global__ __launch_bounds__(64) void delta_scan_kernel(
+    const T* __restrict__ qkv, int C, const float* __restrict__ qn,
+    const float* __restrict__ kn, const float* __restrict__ beta,
+    const float* __restrict__ decay, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ slots, int H, int G, int dk,
+    int dkp, int vd, float* __restrict__ o) {
+  constexpr int COLS = 64 / KS;
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int ks = lane % KS;
+  const int col = blockIdx.z * COLS + lane / KS;
+  const int t0 = cu[b], t1 = cu[b + 1];
+  if (t1 == t0) return;
+  const bool live = col < vd;
+  const int g = h / (H / G);
+  const int64_t slot = slots[b];
+  float* Sp = state + ((slot * H + h) * dk) * vd + (live ? col : 0);
+  float S[DR_ROWS];
+  #pragma unroll
+  for (int r = 0; r < DR_ROWS; ++r) {
+    const int k = ks * DR_ROWS + r;
+    S[r] = (live && k < dk) ? Sp[(int64_t)k * vd] : 0.f;
+  }
+  const int voff = 2 * G * dk + h * vd + (live ? col : 0);
+  for (int t = t0; t < t1; ++t) {
+    const float* kp = kn + ((int64_t)t * G + g) * dkp + ks * DR_ROWS;
+    const float* qp = qn + ((int64_t)t * G + g) * dkp + ks * DR_ROWS;
+    const float dec = decay[(int64_t)t * H + h], bt = beta[(int64_t)t * H + h];
+    const float v = to_f(qkv[(int64_t)t * C + voff]);
+    float kk[DR_ROWS], qq[DR_ROWS];
+    #pragma unroll
+    for (int r = 0; r < DR_ROWS; r += 4) {
+      const float4 k4 = *reinterpret_cast<const float4*>(kp + r);
+      const float4 q4 = *reinterpret_cast<const float4*>(qp + r);
+      kk[r] = k4.x; kk[r + 1] = k4.y; kk[r + 2] = k4.z; kk[r + 3] = k4.w;
+      qq[r] = q4.x; qq[r + 1] = q4.y; qq[r + 2] = q4.z; qq[r + 3] = q4.w;
+    }
+    float sk = 0.f;
+    #pragma unroll
+    for (int r = 0; r < DR_ROWS; ++r) {
+      S[r] *= dec;
+      sk = fmaf(S[r], kk[r], sk);
+    }
+    #pragma unroll
+    for (int off = 1; off < KS; off <<= 1) sk += __shfl_xor(sk, off, SM_WAVE);
+    const float u = bt * (v - sk);
+    float so = 0.f;
+    #pragma unroll
+    for (int r = 0; r < DR_ROWS; ++r) {
+      S[r] = fmaf(kk[r], u, S[r]);
+      so = fmaf(S[r], qq[r], so);
+    }
+    #pragma unroll
+    for (int off = 1; off < KS; off <<= 1) so += __shfl_xor(so, off, SM_WAVE);
+    if (live && ks == 0) o[((int64_t)t * H + h) * vd + col] = so;
+  }
+  #pragma unroll
+  for (int r = 0; r < DR_ROWS; ++r) {
+    const int k = ks * DR_ROWS + r;
+    if (live && k < dk) Sp[(int64_t)k * vd] = S[r];
+  }
+}
+
+// One wave per (token, head).
+template <typename T>
+__global__ __launch_bounds__(64) void delta_finish_kernel(
+    const float* __restrict__ o, const T* __restrict__ gate, int64_t ldg,
+    const float* __restrict__ norm_w, float eps, int H, int vd, T* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* src = o + (t * H + h) * vd;
+  float ss = 0.f;
+  for (int d = lane; d < vd; d += 64) ss += src[d] * src[d];
+  ss = sm_wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vd + eps);
+  for (int d = lane; d < vd; d += 64) {
+    const float gt = to_f(gate[t * ldg + h * vd + d]);
+    out[(t * H + h) * vd + d] = from_f<T>(src[d] * inv * norm_w[d] * (gt * sm_sigmoid(gt)));
+  }
+}
+
+template <typename T>
+void launch_scan(int KS, dim3 grid, hipStream_t stream, const T* qkv, int C, const float* qn,
+                 const float* kn, const float* beta, const float* decay, float* state,
+                 const int* cu, const int* slots, int H, int G, int dk, int dkp, int vd, float* o) {
+#define DR_CASE(N)                                                                       \
+  case N:                                                                                \
+   hipLaunchKernelGGL(( delta_scan_kernel<T, N>), dim3(dim3(grid.x, grid.y, SM_CDIV(vd, 64 / N))), dim3(64), 0, stream,  \
+        qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, dkp, vd, o);            \
+    break;
+  switch (KS) {
+    DR_CASE(1) DR_CASE(2) DR_CASE(4) DR_CASE(8)
+    default: TORCH_CHECK(false, "gated_delta_rule: key dim too large");
+  }
+#undef DR_CASE
+}
+
+}  // namespace
+
+torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Tensor ab,
+                               torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
+                               double eps, torch::Tensor state, torch::Tensor cu,
+                               torch::Tensor slots, int64_t heads, int64_t kv_heads,
+                               int64_t dim, int64_t vdim) {
+  SM_CHECK_CUDA(qkv); SM_CHECK_CUDA(ab); SM_CHECK_F32(ab);
+  SM_CHECK_CUDA(a_log); SM_CHECK_F32(a_log); SM_CHECK_CUDA(dt_bias); SM_CHECK_F32(dt_bias);
+  SM_CHECK_CUDA(onorm_w); SM_CHECK_F32(onorm_w); SM_CHECK_CUDA(state); SM_CHECK_F32(state);
+  SM_CHECK_CUDA(cu); SM_CHECK_I32(cu); SM_CHECK_CUDA(slots); SM_CHECK_I32(slots);
+  const int H = heads, G = kv_heads, dk = dim, vd = vdim;
+  const int64_t T = qkv.size(0);
+  const int C = 2 * G * dk + H * vd;
+  const int B = slots.numel();
+  TORCH_CHECK(G >= 1 && H % G == 0, "gated_delta_rule: heads must be a multiple of kv_heads");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == C, "gated_delta_rule: qkv width");
+  TORCH_CHECK(gate.is_cuda() && gate.dim() == 2 && gate.stride(1) == 1 && gate.size(0) == T &&
+              gate.size(1) == H * vd && gate.scalar_type() == qkv.scalar_type(), "gated_delta_rule: gate layout");
+  TORCH_CHECK(ab.dim() == 2 && ab.size(0) == T && ab.size(1) == 2 * H, "gated_delta_rule: ab is [T, 2H]");
+  TORCH_CHECK(a_log.numel() == H && dt_bias.numel() == H && onorm_w.numel() == vd, "gated_delta_rule: per-head tensors");
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == (int64_t)H * dk * vd && cu.numel() == B + 1,
+              "gated_delta_rule: state/batch layout");
+  int KS = 1;
+  while (KS * DR_ROWS < dk) KS *= 2;
+  TORCH_CHECK(KS <= 8, "gated_delta_rule: key dim above 256");
+  const int dkp = KS * DR_ROWS;
+  auto out = torch::empty({T, (int64_t)H * vd}, qkv.options());
+  if (T == 0 || B == 0) return out;
+  auto f32 = qkv.options().dtype(at::kFloat);
+  auto qn = torch::empty({T, G, dkp}, f32), kn = torch::empty({T, G, dkp}, f32);
+  auto beta = torch::empty({T, H}, f32), decay = torch::empty({T, H}, f32);
+  auto o = torch::empty({T, H, vd}, f32);
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  const bool bf16 = qkv.scalar_type() == at::kBFloat16;
+  if (!bf16) SM_CHECK_F32(qkv);
+  dim3 gscan(B, H), gfin(T, H);
+  if (bf16) {
+    const bf16_t* xp = reinterpret_cast<const bf16_t*>(qkv.data_ptr());
+   hipLaunchKernelGGL(( delta_prepare_kernel<bf16_t>), dim3(T), dim3(256), 0, stream, 
+        xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
+        qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    launch_scan<bf16_t>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+                        beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
+                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, dkp, vd, o.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+   hipLaunchKernelGGL(( delta_finish_kernel<bf16_t>), dim3(gfin), dim3(64), 0, stream, 
+        o.data_ptr<float>(), reinterpret_cast<const bf16_t*>(gate.data_ptr()), gate.stride(0),
+        onorm_w.data_ptr<float>(), (float)eps, H, vd, reinterpret_cast<bf16_t*>(out.data_ptr()));
+  } else {
+    const float* xp = qkv.data_ptr<float>();
+   hipLaunchKernelGGL(( delta_prepare_kernel<float>), dim3(T), dim3(256), 0, stream, 
+        xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
+        qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    launch_scan<float>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+                       beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
+                       cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, dkp, vd, o.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+   hipLaunchKernelGGL(( delta_finish_kernel<float>), dim3(gfin), dim3(64), 0, stream, 
+        o.data_ptr<float>(), gate.data_ptr<float>(), gate.stride(0), onorm_w.data_ptr<float>(),
+        (float)eps, H, vd, out.data_ptr<float>());
+  }
+  SM_CHECK_LAUNCH();
+  return out;
+}

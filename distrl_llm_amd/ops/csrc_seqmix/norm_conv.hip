@@ -1,6 +1,9 @@
 // Offset-weight RMS norm, short causal depthwise convolution with per-slot
-// tails, and the gated parallel-residual update (alone, and fused with the
-// next layer's norm). One workgroup per token row for the row-wise ops.
+// tails (added to its input, or followed by SiLU), the gated
+// parallel-residual update (alone, and fused with the next layer's norm),
+// the sandwich residual update (closing norm of a sublayer, residual sum and
+// the next opening norm in one pass) and the clamped GLU activation. One
+// workgroup per token row for the row-wise ops.
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
 #include "seqmix_common.h"
@@ -58,11 +61,12 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(
   }
 }
 
-// out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j] within the row's
-// sequence; inputs before the portion come from tails[slot].
-template <typename T>
+// acc = sum_j w[:, j] * h[t - taps + 1 + j] within the row's sequence;
+// inputs before the portion come from tails[slot]. ADD_IN: out = h[t] + acc
+// (input rows fp32); SILU: out = acc * sigmoid(acc). h rows are ld apart.
+template <typename Tin, typename T, bool ADD_IN, bool SILU>
 __global__ __launch_bounds__(256) void tap_conv_kernel(
-    const float* __restrict__ h, const float* __restrict__ w,
+    const Tin* __restrict__ h, int64_t ld, const float* __restrict__ w,
     const float* __restrict__ tails, const int* __restrict__ cu,
     const int* __restrict__ tok_seq, const int* __restrict__ slots, int D,
     int taps, T* __restrict__ out) {
@@ -73,21 +77,23 @@ __global__ __launch_bounds__(256) void tap_conv_kernel(
   const int start = cu[b];
   const int rel = t - start;
   const int64_t slot = slots[b];
-  float acc = h[(int64_t)t * D + d];
+  float acc = ADD_IN ? to_f(h[(int64_t)t * ld + d]) : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int src = rel - taps + 1 + j;
     const float v = (src >= 0)
-        ? h[(int64_t)(start + src) * D + d]
+        ? to_f(h[(int64_t)(start + src) * ld + d])
         : tails[(slot * (taps - 1) + (taps - 1 + src)) * D + d];
     acc += w[d * taps + j] * v;
   }
+  if (SILU) acc = acc * sm_sigmoid(acc);
   out[(int64_t)t * D + d] = from_f<T>(acc);
 }
 
 // Advance tails[slot] to the last taps-1 inputs of the row's sequence.
 #define SM_MAX_TAILS 15
+template <typename Tin>
 __global__ __launch_bounds__(256) void tap_tail_kernel(
-    const float* __restrict__ h, float* __restrict__ tails,
+    const Tin* __restrict__ h, int64_t ld, float* __restrict__ tails,
     const int* __restrict__ cu, const int* __restrict__ slots, int D, int taps) {
   const int b = blockIdx.x;
   const int d = blockIdx.y * blockDim.x + threadIdx.x;
@@ -101,13 +107,63 @@ __global__ __launch_bounds__(256) void tap_tail_kernel(
   for (int k = 0; k < SM_MAX_TAILS; ++k) {
     if (k < keep) {
       const int src = n - keep + k;
-      nv[k] = (src >= 0) ? h[(int64_t)(start + src) * D + d]
+      nv[k] = (src >= 0) ? to_f(h[(int64_t)(start + src) * ld + d])
                          : tails[(slot * keep + (k + n)) * D + d];
     }
   }
   #pragma unroll
   for (int k = 0; k < SM_MAX_TAILS; ++k)
     if (k < keep) tails[(slot * keep + k) * D + d] = nv[k];
+}
+
+// x += s / sqrt(mean(s^2) + eps) * (1 + post_w), s = y (+ y2); then, with
+// next_w, h = x / sqrt(mean(x^2) + eps) * (1 + next_w). y and y2 are bf16 or
+// fp32 each (flags), h is T.
+SM_INLINE float ld_any(const void* p, bool is_bf16, int64_t i) {
+  return is_bf16 ? __bfloat162float(reinterpret_cast<const bf16_t*>(p)[i])
+                 : reinterpret_cast<const float*>(p)[i];
+}
+template <typename T>
+__global__ __launch_bounds__(256) void sandwich_residual_kernel(
+    float* __restrict__ x, const void* __restrict__ y, bool y_bf16,
+    const void* __restrict__ y2, bool y2_bf16, const float* __restrict__ post_w,
+    const float* __restrict__ next_w, float eps, int D, T* __restrict__ h) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float s = ld_any(y, y_bf16, row * D + d);
+    if (y2 != nullptr) s += ld_any(y2, y2_bf16, row * D + d);
+    ss += s * s;
+  }
+  ss = sm_block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+  float xx = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float s = ld_any(y, y_bf16, row * D + d);
+    if (y2 != nullptr) s += ld_any(y2, y2_bf16, row * D + d);
+    const float v = x[row * D + d] + s * inv * (1.0f + post_w[d]);
+    x[row * D + d] = v;
+    xx += v * v;
+  }
+  if (next_w == nullptr) return;
+  xx = sm_block_sum(xx, red);   // also orders the row's writes before the re-read
+  const float inv2 = 1.0f / sqrtf(xx / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += blockDim.x)
+    h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (1.0f + next_w[d]));
+}
+
+// gu rows = [gate (ff) | up (ff)]: g = min(gate, limit), u = clamp(up, +-limit),
+// out = g * sigmoid(1.702 g) * (u + 1).
+template <typename T>
+__global__ __launch_bounds__(256) void capped_glu_kernel(
+    const T* __restrict__ gu, int64_t n, int ff, float limit, T* __restrict__ out) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= n) return;
+  const int64_t t = id / ff;
+  const int f = id % ff;
+  out[id] = from_f<T>(sm_capped_glu(to_f(gu[t * 2 * ff + f]),
+                                    to_f(gu[t * 2 * ff + ff + f]), limit));
 }
 
 }  // namespace
@@ -216,21 +272,134 @@ torch::Tensor causal_tap_conv(torch::Tensor h, torch::Tensor w, torch::Tensor ta
   auto stream = at::cuda::getCurrentCUDAStream();
   dim3 grid(T, SM_CDIV(D, 256));
   if (out_bf16)
-    tap_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>(
-        h.data_ptr<float>(), w.data_ptr<float>(), tails.data_ptr<float>(),
+    tap_conv_kernel<float, bf16_t, true, false><<<grid, 256, 0, stream>>>(
+        h.data_ptr<float>(), (int64_t)D, w.data_ptr<float>(), tails.data_ptr<float>(),
         cu.data_ptr<int>(), tok_seq.data_ptr<int>(), slots.data_ptr<int>(), D, taps,
         reinterpret_cast<bf16_t*>(out.data_ptr()));
   else
-    tap_conv_kernel<float><<<grid, 256, 0, stream>>>(
-        h.data_ptr<float>(), w.data_ptr<float>(), tails.data_ptr<float>(),
+    tap_conv_kernel<float, float, true, false><<<grid, 256, 0, stream>>>(
+        h.data_ptr<float>(), (int64_t)D, w.data_ptr<float>(), tails.data_ptr<float>(),
         cu.data_ptr<int>(), tok_seq.data_ptr<int>(), slots.data_ptr<int>(), D, taps,
         out.data_ptr<float>());
   SM_CHECK_LAUNCH();
   if (taps > 1) {
     dim3 g2(B, SM_CDIV(D, 256));
-    tap_tail_kernel<<<g2, 256, 0, stream>>>(h.data_ptr<float>(), tails.data_ptr<float>(),
-                                            cu.data_ptr<int>(), slots.data_ptr<int>(), D, taps);
+    tap_tail_kernel<float><<<g2, 256, 0, stream>>>(h.data_ptr<float>(), (int64_t)D,
+                                                   tails.data_ptr<float>(), cu.data_ptr<int>(),
+                                                   slots.data_ptr<int>(), D, taps);
     SM_CHECK_LAUNCH();
   }
+  return out;
+}
+
+torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tails,
+                            torch::Tensor cu, torch::Tensor tok_seq,
+                            torch::Tensor slots, bool out_bf16) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1, "tap_conv_silu: x must be row-major");
+  SM_CHECK_CUDA(w); SM_CHECK_F32(w); SM_CHECK_CUDA(tails); SM_CHECK_F32(tails);
+  SM_CHECK_CUDA(cu); SM_CHECK_I32(cu); SM_CHECK_CUDA(tok_seq); SM_CHECK_I32(tok_seq);
+  SM_CHECK_CUDA(slots); SM_CHECK_I32(slots);
+  const int64_t T = x.size(0);
+  const int C = x.size(1);
+  const int64_t ld = x.stride(0);
+  const int taps = w.size(1);
+  const int B = slots.numel();
+  const bool in_bf16 = x.scalar_type() == at::kBFloat16;
+  TORCH_CHECK(in_bf16 || x.scalar_type() == at::kFloat, "tap_conv_silu: dtype");
+  TORCH_CHECK(in_bf16 == out_bf16, "tap_conv_silu: output dtype follows the input");
+  TORCH_CHECK(w.size(0) == C && taps >= 1 && taps - 1 <= SM_MAX_TAILS, "tap_conv_silu: weight shape");
+  TORCH_CHECK(tails.dim() == 3 && tails.size(1) == taps - 1 && tails.size(2) == C, "tap_conv_silu: tails shape");
+  TORCH_CHECK(cu.numel() == B + 1 && tok_seq.numel() == T, "tap_conv_silu: batch layout");
+  auto out = torch::empty({T, C}, x.options());
+  if (T == 0) return out;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  dim3 grid(T, SM_CDIV(C, 256)), g2(B, SM_CDIV(C, 256));
+  if (in_bf16) {
+    const bf16_t* xp = reinterpret_cast<const bf16_t*>(x.data_ptr());
+    tap_conv_kernel<bf16_t, bf16_t, false, true><<<grid, 256, 0, stream>>>(
+        xp, ld, w.data_ptr<float>(), tails.data_ptr<float>(), cu.data_ptr<int>(),
+        tok_seq.data_ptr<int>(), slots.data_ptr<int>(), C, taps,
+        reinterpret_cast<bf16_t*>(out.data_ptr()));
+    SM_CHECK_LAUNCH();
+    if (taps > 1)
+      tap_tail_kernel<bf16_t><<<g2, 256, 0, stream>>>(xp, ld, tails.data_ptr<float>(),
+                                                      cu.data_ptr<int>(), slots.data_ptr<int>(), C, taps);
+  } else {
+    tap_conv_kernel<float, float, false, true><<<grid, 256, 0, stream>>>(
+        x.data_ptr<float>(), ld, w.data_ptr<float>(), tails.data_ptr<float>(), cu.data_ptr<int>(),
+        tok_seq.data_ptr<int>(), slots.data_ptr<int>(), C, taps, out.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    if (taps > 1)
+      tap_tail_kernel<float><<<g2, 256, 0, stream>>>(x.data_ptr<float>(), ld, tails.data_ptr<float>(),
+                                                     cu.data_ptr<int>(), slots.data_ptr<int>(), C, taps);
+  }
+  SM_CHECK_LAUNCH();
+  return out;
+}
+
+c10::optional<torch::Tensor> sandwich_residual_norm(
+    torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2,
+    torch::Tensor post_w, c10::optional<torch::Tensor> next_w, double eps,
+    bool out_bf16) {
+  SM_CHECK_CUDA(x); SM_CHECK_F32(x); SM_CHECK_CUDA(y); SM_CHECK_CUDA(post_w); SM_CHECK_F32(post_w);
+  const int64_t T = x.size(0);
+  const int D = x.size(1);
+  auto kind = [](const torch::Tensor& t) {
+    TORCH_CHECK(t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat,
+                "sandwich_residual_norm: addends are bf16 or fp32");
+    return t.scalar_type() == at::kBFloat16;
+  };
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == T && y.size(1) == D && post_w.numel() == D,
+              "sandwich_residual_norm: shapes");
+  const bool yb = kind(y);
+  const void* y2p = nullptr;
+  bool y2b = false;
+  if (y2.has_value()) {
+    SM_CHECK_CUDA(*y2);
+    TORCH_CHECK(y2->dim() == 2 && y2->size(0) == T && y2->size(1) == D, "sandwich_residual_norm: y2 shape");
+    y2b = kind(*y2);
+    y2p = y2->data_ptr();
+  }
+  const float* nw = nullptr;
+  c10::optional<torch::Tensor> h;
+  if (next_w.has_value()) {
+    SM_CHECK_CUDA(*next_w); SM_CHECK_F32(*next_w);
+    TORCH_CHECK(next_w->numel() == D, "sandwich_residual_norm: norm weight");
+    nw = next_w->data_ptr<float>();
+    h = torch::empty({T, D}, x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  }
+  if (T == 0) return h;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  if (out_bf16)
+    sandwich_residual_kernel<bf16_t><<<T, 256, 0, stream>>>(
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps, D,
+        h.has_value() ? reinterpret_cast<bf16_t*>(h->data_ptr()) : nullptr);
+  else
+    sandwich_residual_kernel<float><<<T, 256, 0, stream>>>(
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps, D,
+        h.has_value() ? h->data_ptr<float>() : nullptr);
+  SM_CHECK_LAUNCH();
+  return h;
+}
+
+torch::Tensor capped_glu(torch::Tensor gu, double limit) {
+  SM_CHECK_CUDA(gu);
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0, "capped_glu: rows are [gate | up]");
+  const int64_t T = gu.size(0);
+  const int ff = gu.size(1) / 2;
+  auto out = torch::empty({T, ff}, gu.options());
+  const int64_t n = T * ff;
+  if (n == 0) return out;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  if (gu.scalar_type() == at::kBFloat16)
+    capped_glu_kernel<bf16_t><<<SM_CDIV(n, 256), 256, 0, stream>>>(
+        reinterpret_cast<const bf16_t*>(gu.data_ptr()), n, ff, (float)limit,
+        reinterpret_cast<bf16_t*>(out.data_ptr()));
+  else {
+    SM_CHECK_F32(gu);
+    capped_glu_kernel<float><<<SM_CDIV(n, 256), 256, 0, stream>>>(
+        gu.data_ptr<float>(), n, ff, (float)limit, out.data_ptr<float>());
+  }
+  SM_CHECK_LAUNCH();
   return out;
 }

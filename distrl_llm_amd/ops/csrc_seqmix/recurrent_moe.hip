@@ -1,7 +1,10 @@
 // minGRU scan over a flat varlen batch (fp32 state per slot), the fp32
-// top-k router, and the mixture-of-experts feed-forward as two grouped
-// GEMMs over expert-sorted rows (bf16: MFMA 16x16x32 tiles; fp32: plain
-// FMA) followed by a fixed-order weighted combine.
+// top-k routers (softmax over the chosen logits; or softmax over every
+// output with a choice correction and scaled, unnormalised weights), and the
+// mixture-of-experts feed-forward as two grouped GEMMs over expert-sorted
+// rows (bf16: MFMA 16x16x32 tiles; fp32: plain FMA; SiLU-gated or clamped
+// GLU experts) followed by a fixed-order weighted combine, which also adds
+// the identity experts' share of the input.
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
 #include "seqmix_common.h"
@@ -116,13 +119,17 @@ __global__ __launch_bounds__(256) void mingru_chunk_apply_kernel(
 // One workgroup per token: the waves share the experts' fp32 logits, then
 // one lane picks the top-k by repeated arg-max (ties: the lowest index) and
 // takes the softmax over the chosen logits.
+// ALL: scores s = softmax over all E outputs (no bias); the top-k of
+// s + corr are chosen; weights = s[chosen] * wscale, not renormalised.
 #define SM_MAX_EXPERTS 256
-template <typename T>
+template <typename T, bool ALL>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ w,
     const float* __restrict__ bias, int D, int E, int top,
-    int* __restrict__ idx, float* __restrict__ wts) {
+    int* __restrict__ idx, float* __restrict__ wts,
+    const float* __restrict__ corr, float wscale) {
   __shared__ float z[SM_MAX_EXPERTS];
+  __shared__ float sc[SM_MAX_EXPERTS];
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int e = wave; e < E; e += 4) {
@@ -137,9 +144,34 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
     }
     for (; d < D; d += 64) a0 = fmaf(to_f(h[t * D + d]), we[d], a0);
     const float acc = sm_wave_sum((a0 + a1) + (a2 + a3));
-    if (lane == 0) z[e] = acc + bias[e];
+    if (lane == 0) z[e] = acc + (bias != nullptr ? bias[e] : 0.f);
   }
   __syncthreads();
+  if (ALL) {
+    if (threadIdx.x == 0) {
+      float vmax = -INFINITY, sum = 0.f;
+      for (int e = 0; e < E; ++e) vmax = fmaxf(vmax, z[e]);
+      for (int e = 0; e < E; ++e) {
+        sc[e] = expf(z[e] - vmax);
+        sum += sc[e];
+      }
+      for (int e = 0; e < E; ++e) {
+        sc[e] /= sum;
+        z[e] = sc[e] + (corr != nullptr ? corr[e] : 0.f);
+      }
+      for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bv = -INFINITY;
+        for (int e = 0; e < E; ++e)
+          if (z[e] > bv) { bv = z[e]; best = e; }
+        if (best < 0) best = 0;
+        idx[t * top + k] = best;
+        wts[t * top + k] = sc[best] * wscale;
+        z[best] = -INFINITY;
+      }
+    }
+    return;
+  }
   if (threadIdx.x == 0) {
     float vmax = 0.f, sum = 0.f;
     for (int k = 0; k < top; ++k) {
@@ -162,12 +194,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 // Group the (token, choice) pairs by expert in one workgroup: off[e] = first
 // sorted row of expert e, src[row] = token of that row, inv[pair] = its row.
 // The order inside an expert is arbitrary; every row's result is independent
-// of it and the combine reads rows back through inv.
+// of it and the combine reads rows back through inv. Called with E = weight
+// sets + 1: indices at or above the weight sets (identity experts) share the
+// last bin, whose rows no GEMM touches.
 __global__ __launch_bounds__(1024) void moe_group_kernel(
     const int* __restrict__ idx, int M, int top, int E, int* __restrict__ off,
     int* __restrict__ src, int* __restrict__ inv) {
-  __shared__ int cnt[SM_MAX_EXPERTS];
-  __shared__ int start[SM_MAX_EXPERTS + 1];
+  __shared__ int cnt[SM_MAX_EXPERTS + 1];
+  __shared__ int start[SM_MAX_EXPERTS + 2];
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < M; i += blockDim.x)
@@ -197,11 +231,15 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(
 // Rows are sorted by expert: expert e owns rows off[e]..off[e+1]. A
 // workgroup (4 waves) computes a 64-row x 64-column tile of one expert;
 // wave w owns columns w*16..w*16+15 for the four 16-row m-tiles.
-// MODE 0: out[i, f] = silu(a_i . Wg[f]) * (a_i . Wu[f]), a_i = A[src[i]],
+// MODE 0: out[i, f] = act(a_i . Wg[f], a_i . Wu[f]), a_i = A[src[i]],
+//         act(g, u) = silu(g) u (limit 0) or the clamped GLU (limit > 0);
 //         W[e] = [gate (N rows); up (N rows)] x K;   out bf16 [M, N]
 // MODE 1: out[i, n] = a_i . W[e][n], a_i = A[i];     out fp32 [M, N]
 // MFMA 16x16x32 bf16 fragments: A lane l -> row l&15, k (l>>4)*8..+7;
 // B lane l -> column l&15, same k; D lane l reg r -> row (l>>4)*4+r, col l&15.
+SM_INLINE float moe_act(float g, float u, float limit) {
+  return (limit > 0.f) ? sm_capped_glu(g, u, limit) : g * sm_sigmoid(g) * u;
+}
 SM_INLINE bf16v8 load8(const bf16_t* p, int valid, bool vec) {
   bf16v8 v;
   if (vec && valid >= 8) {
@@ -224,7 +262,7 @@ template <int MODE, int MT, int NWV>
 __global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const int* __restrict__ src,
     const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
-    int K, void* __restrict__ outp) {
+    int K, void* __restrict__ outp, float limit) {
   constexpr int BM = 16 * MT;
   __shared__ __attribute__((aligned(16))) bf16_t a_lds[BM * GG_LD];
   // which expert / row range is this tile?
@@ -296,8 +334,8 @@ __global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
       if (r < rows) {
         const int64_t o = (int64_t)(row0 + r) * N + n;
         if (MODE == 0) {
-          const float g = acc[mt][rr];
-          reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(g * sm_sigmoid(g) * acc2[mt][rr]);
+          reinterpret_cast<bf16_t*>(outp)[o] =
+              __float2bfloat16(moe_act(acc[mt][rr], acc2[mt][rr], limit));
         } else {
           reinterpret_cast<float*>(outp)[o] = acc[mt][rr];
         }
@@ -315,7 +353,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_splitk_kernel(
     const bf16_t* __restrict__ A, const int* __restrict__ src,
     const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
-    int K, void* __restrict__ outp) {
+    int K, void* __restrict__ outp, float limit) {
   __shared__ float red[3][64][8];
   int e = -1, row0 = 0, rows = 0, tiles = 0;
   for (int i = 0; i < E; ++i) {
@@ -373,7 +411,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_splitk_kernel(
     if (r < rows) {
       const int64_t o = (int64_t)(row0 + r) * N + n;
       if (MODE == 0)
-        reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(g * sm_sigmoid(g) * u);
+        reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(moe_act(g, u, limit));
       else
         reinterpret_cast<float*>(outp)[o] = g;
     }
@@ -386,10 +424,11 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
     const float* __restrict__ A, const int* __restrict__ src,
     const float* __restrict__ W, const int* __restrict__ off, int E, int M,
-    int N, int K, float* __restrict__ out) {
+    int N, int K, float* __restrict__ out, float limit) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= (int64_t)M * N) return;
   const int i = id / N, n = id % N;
+  if (i >= off[E]) return;                 // rows of identity experts
   int e = 0;
   while (e + 1 < E && i >= off[e + 1]) ++e;
   const int Nw = (MODE == 0) ? 2 * N : N;
@@ -400,18 +439,24 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
     g = fmaf(a[k], wg[k], g);
     if (MODE == 0) u = fmaf(a[k], wg[(int64_t)N * K + k], u);
   }
-  out[id] = (MODE == 0) ? g * sm_sigmoid(g) * u : g;
+  out[id] = (MODE == 0) ? moe_act(g, u, limit) : g;
 }
 
-// out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order)
+// out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order); a
+// choice at or above E is an identity expert: its output is the input row.
+template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const float* __restrict__ y, const int* __restrict__ inv,
-    const float* __restrict__ wts, int top, int D, float* __restrict__ out) {
+    const float* __restrict__ wts, const int* __restrict__ idx,
+    const T* __restrict__ h, int E, int top, int D, float* __restrict__ out) {
   const int64_t t = blockIdx.x;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float acc = 0.f;
-    for (int k = 0; k < top; ++k)
-      acc += wts[t * top + k] * y[(int64_t)inv[t * top + k] * D + d];
+    for (int k = 0; k < top; ++k) {
+      const float v = (idx[t * top + k] >= E) ? to_f(h[t * D + d])
+                                              : y[(int64_t)inv[t * top + k] * D + d];
+      acc += wts[t * top + k] * v;
+    }
     out[t * D + d] = acc;
   }
 }
@@ -484,35 +529,57 @@ torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor s
   return out;
 }
 
-std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
-                                     torch::Tensor router_b, int64_t top) {
+static std::vector<torch::Tensor> moe_route_impl(
+    torch::Tensor h, torch::Tensor router_w, c10::optional<torch::Tensor> router_b,
+    int64_t top, bool all, c10::optional<torch::Tensor> corr, double wscale) {
   SM_CHECK_CUDA(h); SM_CHECK_CUDA(router_w); SM_CHECK_F32(router_w);
-  SM_CHECK_CUDA(router_b); SM_CHECK_F32(router_b);
   const int64_t T = h.size(0);
   const int D = h.size(1);
   const int E = router_w.size(0);
-  TORCH_CHECK(router_w.size(1) == D && router_b.numel() == E, "moe_route: shapes");
+  TORCH_CHECK(router_w.size(1) == D, "moe_route: shapes");
   TORCH_CHECK(E <= SM_MAX_EXPERTS && top >= 1 && top <= E, "moe_route: experts/top");
+  const float* bp = nullptr;
+  const float* cp = nullptr;
+  if (router_b.has_value()) {
+    SM_CHECK_CUDA(*router_b); SM_CHECK_F32(*router_b);
+    TORCH_CHECK(router_b->numel() == E, "moe_route: bias shape");
+    bp = router_b->data_ptr<float>();
+  }
+  if (corr.has_value()) {
+    SM_CHECK_CUDA(*corr); SM_CHECK_F32(*corr);
+    TORCH_CHECK(corr->numel() == E, "moe_route: correction shape");
+    cp = corr->data_ptr<float>();
+  }
   auto idx = torch::empty({T, top}, h.options().dtype(at::kInt));
   auto wts = torch::empty({T, top}, h.options().dtype(at::kFloat));
   if (T == 0) return {idx, wts};
   auto stream = at::cuda::getCurrentCUDAStream();
-  if (h.scalar_type() == at::kBFloat16)
-    moe_route_kernel<bf16_t><<<T, 256, 0, stream>>>(
-        reinterpret_cast<const bf16_t*>(h.data_ptr()), router_w.data_ptr<float>(),
-        router_b.data_ptr<float>(), D, E, (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
-  else {
-    SM_CHECK_F32(h);
-    moe_route_kernel<float><<<T, 256, 0, stream>>>(
-        h.data_ptr<float>(), router_w.data_ptr<float>(), router_b.data_ptr<float>(), D, E,
-        (int)top, idx.data_ptr<int>(), wts.data_ptr<float>());
-  }
+  const bool bf16 = h.scalar_type() == at::kBFloat16;
+  if (!bf16) SM_CHECK_F32(h);
+#define ROUTE(TY, ALLV)                                                                    \
+  moe_route_kernel<TY, ALLV><<<T, 256, 0, stream>>>(                                       \
+      reinterpret_cast<const TY*>(h.data_ptr()), router_w.data_ptr<float>(), bp, D, E,     \
+      (int)top, idx.data_ptr<int>(), wts.data_ptr<float>(), cp, (float)wscale)
+  if (bf16) { if (all) ROUTE(bf16_t, true); else ROUTE(bf16_t, false); }
+  else { if (all) ROUTE(float, true); else ROUTE(float, false); }
+#undef ROUTE
   SM_CHECK_LAUNCH();
   return {idx, wts};
 }
 
-torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
-                          torch::Tensor exp_gu, torch::Tensor exp_down) {
+std::vector<torch::Tensor> moe_route(torch::Tensor h, torch::Tensor router_w,
+                                     torch::Tensor router_b, int64_t top) {
+  return moe_route_impl(h, router_w, router_b, top, false, c10::nullopt, 1.0);
+}
+
+std::vector<torch::Tensor> moe_route_all(torch::Tensor h, torch::Tensor router_w,
+                                         c10::optional<torch::Tensor> correction,
+                                         int64_t top, double scale) {
+  return moe_route_impl(h, router_w, c10::nullopt, top, true, correction, scale);
+}
+
+static torch::Tensor moe_experts_impl(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                                      torch::Tensor exp_gu, torch::Tensor exp_down, float limit) {
   SM_CHECK_CUDA(h); SM_CHECK_CUDA(idx); SM_CHECK_I32(idx); SM_CHECK_CUDA(wts); SM_CHECK_F32(wts);
   SM_CHECK_CUDA(exp_gu); SM_CHECK_CUDA(exp_down);
   const int64_t T = h.size(0);
@@ -532,11 +599,11 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
   const int64_t M = T * top;
   // group the (token, choice) pairs by expert on the device (no host sync)
   auto iopt = h.options().dtype(at::kInt);
-  auto off = torch::empty({E + 1}, iopt);
+  auto off = torch::empty({E + 2}, iopt);    // E weight sets + the identity bin
   auto src = torch::empty({M}, iopt);
   auto inv = torch::empty({M}, iopt);
   auto stream = at::cuda::getCurrentCUDAStream();
-  moe_group_kernel<<<1, 1024, 0, stream>>>(idx.data_ptr<int>(), (int)M, top, E,
+  moe_group_kernel<<<1, 1024, 0, stream>>>(idx.data_ptr<int>(), (int)M, top, E + 1,
                                            off.data_ptr<int>(), src.data_ptr<int>(),
                                            inv.data_ptr<int>());
   SM_CHECK_LAUNCH();
@@ -550,20 +617,20 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
       // a few rows per expert (decoding): 16x16 tiles, K split over four waves
       const int row_tiles = SM_CDIV(M, 16) + E;
       moe_gemm_bf16_splitk_kernel<0><<<dim3(row_tiles, SM_CDIV(ff, 16)), 256, 0, stream>>>(
-          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr());
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit);
       SM_CHECK_LAUNCH();
       moe_gemm_bf16_splitk_kernel<1><<<dim3(row_tiles, SM_CDIV(D, 16)), 256, 0, stream>>>(
           reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
-          D, ff, y.data_ptr());
+          D, ff, y.data_ptr(), 0.f);
       SM_CHECK_LAUNCH();
     } else {
       const int row_tiles = SM_CDIV(M, 64) + E;
       moe_gemm_bf16_kernel<0, 4, 4><<<dim3(row_tiles, SM_CDIV(ff, 64)), 256, 0, stream>>>(
-          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr());
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit);
       SM_CHECK_LAUNCH();
       moe_gemm_bf16_kernel<1, 4, 4><<<dim3(row_tiles, SM_CDIV(D, 64)), 256, 0, stream>>>(
           reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
-          D, ff, y.data_ptr());
+          D, ff, y.data_ptr(), 0.f);
       SM_CHECK_LAUNCH();
     }
   } else {
@@ -571,15 +638,32 @@ torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
     auto act = torch::empty({M, ff}, h.options());
     moe_gemm_f32_kernel<0><<<SM_CDIV(M * ff, 256), 256, 0, stream>>>(
         h.data_ptr<float>(), src.data_ptr<int>(), exp_gu.data_ptr<float>(),
-        off.data_ptr<int>(), E, (int)M, ff, D, act.data_ptr<float>());
+        off.data_ptr<int>(), E, (int)M, ff, D, act.data_ptr<float>(), limit);
     SM_CHECK_LAUNCH();
     moe_gemm_f32_kernel<1><<<SM_CDIV(M * D, 256), 256, 0, stream>>>(
         act.data_ptr<float>(), nullptr, exp_down.data_ptr<float>(), off.data_ptr<int>(), E,
-        (int)M, D, ff, y.data_ptr<float>());
+        (int)M, D, ff, y.data_ptr<float>(), 0.f);
     SM_CHECK_LAUNCH();
   }
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y.data_ptr<float>(), inv.data_ptr<int>(),
-                                            wts.data_ptr<float>(), top, D, out.data_ptr<float>());
+  if (h.scalar_type() == at::kBFloat16)
+    moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>(
+        y.data_ptr<float>(), inv.data_ptr<int>(), wts.data_ptr<float>(), idx.data_ptr<int>(),
+        reinterpret_cast<const bf16_t*>(h.data_ptr()), E, top, D, out.data_ptr<float>());
+  else
+    moe_combine_kernel<float><<<T, 256, 0, stream>>>(
+        y.data_ptr<float>(), inv.data_ptr<int>(), wts.data_ptr<float>(), idx.data_ptr<int>(),
+        h.data_ptr<float>(), E, top, D, out.data_ptr<float>());
   SM_CHECK_LAUNCH();
   return out;
+}
+
+torch::Tensor moe_experts(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                          torch::Tensor exp_gu, torch::Tensor exp_down) {
+  return moe_experts_impl(h, idx, wts, exp_gu, exp_down, 0.f);
+}
+
+torch::Tensor moe_experts_glu(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                              torch::Tensor exp_gu, torch::Tensor exp_down, double limit) {
+  TORCH_CHECK(limit > 0, "moe_experts_glu: the clamp limit must be positive");
+  return moe_experts_impl(h, idx, wts, exp_gu, exp_down, (float)limit);
 }

@@ -41,6 +41,12 @@ SM_INLINE float sm_block_sum(float x, float* red) {
   return r;
 }
 SM_INLINE float sm_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+// clamped GLU: g = min(gate, limit), u = clamp(up, +-limit), g sigmoid(1.702 g) (u + 1)
+SM_INLINE float sm_capped_glu(float g, float u, float limit) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g * sm_sigmoid(1.702f * g) * (u + 1.0f);
+}
 
 #define SM_CHECK_LAUNCH()                                                  \
   do {                                                                     \

@@ -154,12 +154,11 @@ def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
 def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
     """Fused sublayer tail: x += rms_unit(y [+ y2]) * (1 + post_w) on the
     fp32 residual (in place), then, with ``next_w``, the next offset RMS
-    norm of the new residual -> (fp32, out_dtype); None without."""
+    norm of the new residual in ``out_dtype``; None without."""
     if x.is_cuda:
-        r = _ext("sandwich_residual_norm").sandwich_residual_norm(
+        return _ext("sandwich_residual_norm").sandwich_residual_norm(
             x, y.contiguous(), None if y2 is None else y2.contiguous(), post_w,
             next_w, eps, _bf16(out_dtype))
-        return None if next_w is None else r
     return R.sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype)
 
 

@@ -187,13 +187,13 @@ def gated_residual_add(x, mix, ff, gates, gate_b, mult):
 def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
     """x += rms_unit(y [+ y2]) * (1 + post_w) on the fp32 residual, in
     place; with ``next_w`` also returns the next offset RMS norm of the new
-    residual as (fp32, out_dtype), else None."""
+    residual in ``out_dtype``, else None."""
     s = y.float() if y2 is None else y.float() + y2.float()
     x.add_(s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps)
            * (1.0 + post_w.float()))
     if next_w is None:
         return None
-    return offset_rmsnorm(x, next_w, eps, out_dtype)
+    return offset_rmsnorm(x, next_w, eps, out_dtype)[1]
 
 
 def _rotate_pairs(v, positions, base, dims):
