@@ -546,9 +546,10 @@ def nedasun_spec_from_config(cfg: dict, name: str = "nedasun") -> HybridSpec:
                 raise ValueError(f"layer {i}: rot.dims must be even and <= dim")
             if mixes and v_first is None:
                 v_first = i
-            elif mixes and layers[v_first].mixer.v_size != mixer.v_size:
+            elif mixes and ((layers[v_first].mixer.kv_heads, layers[v_first].mixer.vdim)
+                            != (kvh, mixer.vdim)):
                 raise ValueError(f"layer {i}: value mixing needs the first "
-                                 f"mixing layer's kv_heads * vdim")
+                                 f"mixing layer's kv_heads and vdim")
         elif lc["type"] == "delta":
             mixer = DeltaRuleSpec(heads=heads, kv_heads=kvh, dim=int(mc["dim"]),
                                   vdim=int(mc["vdim"]), taps=int(mc["conv"]))

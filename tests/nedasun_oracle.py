@@ -286,3 +286,37 @@ def random_weights(cfg, seed=0, round_bf16=True):
             r = 0.1 * r
         W[name] = r.to(torch.bfloat16).float() if round_bf16 else r
     return W
+
+
+# ------------------------------------------------------- config builders
+
+def attn_layer(heads=4, kv_heads=2, dim=8, vdim=6, rot_dims=None, base=10000.0,
+               scale=None, softcap=5.0, v_mix=True, mlp="dense"):
+    mc = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+          "scale": dim ** -0.5 if scale is None else scale, "softcap": softcap,
+          "rot": {"base": base, "dims": dim if rot_dims is None else rot_dims},
+          "v_mix": v_mix}
+    return {"type": "attention", "mixer": mc, "mlp": mlp_cfg(mlp)}
+
+
+def delta_layer(heads=4, kv_heads=2, dim=8, vdim=6, conv=3, mlp="moe"):
+    mc = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+    return {"type": "delta", "mixer": mc, "mlp": mlp_cfg(mlp)}
+
+
+def mlp_cfg(kind, **kw):
+    if kind is None or isinstance(kind, dict):
+        return kind
+    if kind == "dense":
+        return {"kind": "dense", "ff": kw.get("ff", 24), "limit": kw.get("limit", 0.8)}
+    return {"kind": "moe",
+            "expert": {"ff": kw.get("ff", 10), "limit": kw.get("limit", 0.6)},
+            "router": {"experts": kw.get("experts", 5), "identity": kw.get("identity", 1),
+                       "scale": kw.get("scale", 1.7), "top": kw.get("top", 2)},
+            "shared": ({"ff": kw.get("shared_ff", 12), "limit": kw.get("shared_limit", 0.9)}
+                       if kw.get("shared", True) else None)}
+
+
+def make_cfg(layers, width=16, vocab=41, eps=1e-5):
+    return {"architecture": "Nedasun", "layers": layers, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}
