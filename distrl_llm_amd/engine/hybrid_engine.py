@@ -73,7 +73,9 @@ class _DecodeGraph:
                     cu=list(range(self.rows + 1)),
                     slots=slots + [eng.slots.scratch_slot] * pad,
                     block_tables=tables + [[scratch]] * pad,
-                    tiles=[(b, b, 1) for b in range(self.rows)], max_tile=1)
+                    tiles=[(b, b, 1) for b in range(self.rows)], max_tile=1,
+                    wide_tiles=[(b, b, 1) for b in range(self.rows)],
+                    max_wide_tile=1)
         return eng._pack(tokens + [0] * pad, meta, list(range(self.rows)),
                          max_nb=self.max_nb)
 
@@ -221,11 +223,13 @@ class HybridEngine:
                 want_rows.append(base + w)
         lengths = [len(t) for _, t in work]
         tiles, max_tile = SM.query_tiles(lengths)
+        wide, max_wide = SM.query_tiles(lengths, SM.WIDE_QUERY_TILE)
         chunks, chunk_cu = SM.scan_chunks(lengths)
         meta = dict(positions=positions, tok_seq=tok_seq, page_slot=page_slot,
                     cu=cu, slots=slot_idx,
                     block_tables=[q.block_table for q, _ in work],
-                    tiles=tiles, max_tile=max_tile, scan_chunks=chunks,
+                    tiles=tiles, max_tile=max_tile, wide_tiles=wide,
+                    max_wide_tile=max_wide, scan_chunks=chunks,
                     scan_cu=chunk_cu)
         return tokens, meta, want_rows
 
@@ -243,13 +247,17 @@ class HybridEngine:
                            ("tok_seq", meta["tok_seq"]),
                            ("page_slot", meta["page_slot"]), ("cu", meta["cu"]),
                            ("slots", meta["slots"]), ("block_tables", tables),
-                           ("tiles", tiles), ("want", want_rows),
+                           ("tiles", tiles),
+                           ("wide_tiles", [v for t in meta.get("wide_tiles", [])
+                                           for v in t]),
+                           ("want", want_rows),
                            ("scan_chunks", [v for c in meta.get("scan_chunks", [])
                                             for v in c]),
                            ("scan_cu", meta.get("scan_cu", []))):
             lay[name] = (len(flat), len(vals))
             flat.extend(vals)
         lay["max_nb"] = max_nb
+        lay["max_wide_tile"] = meta.get("max_wide_tile", 1)
         return flat, lay
 
     @staticmethod
@@ -261,6 +269,8 @@ class HybridEngine:
                                     "slots")}
         meta["block_tables"] = cut("block_tables").view(-1, lay["max_nb"])
         meta["tiles"] = cut("tiles").view(-1, 3)
+        meta["wide_tiles"] = cut("wide_tiles").view(-1, 3)
+        meta["max_wide_tile"] = lay["max_wide_tile"]
         meta["scan_chunks"] = cut("scan_chunks").view(-1, 3)
         meta["scan_cu"] = cut("scan_cu")
         meta["max_tile"] = max_tile
@@ -342,7 +352,8 @@ class HybridEngine:
                               meta["block_tables"], self.pool.block_size,
                               meta["cu"], meta["tok_seq"], meta["positions"],
                               m.scale, m.softcap, L.sink, L.talk, self.dtype,
-                              tiles=meta["tiles"], max_tile=meta["max_tile"])
+                              tiles=meta["wide_tiles"],
+                              max_tile=meta["max_wide_tile"])
         return F.linear(o, L.out_w)
 
     def _mix_delta(self, i, m, L, hm, meta):

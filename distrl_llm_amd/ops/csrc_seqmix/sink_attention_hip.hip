@@ -263,7 +263,7 @@ torch::Tensor sink_attention(torch::Tensor q, torch::Tensor cache, int64_t heads
   const bool bf16 = q.scalar_type() == at::kBFloat16;
   if (bf16 && tiles.has_value() && max_tile_queries > 1 && sink_attention_mfma_fits(dk, vd, G, all_groups)) {
     SM_CHECK_CUDA(*tiles); SM_CHECK_I32(*tiles);
-    TORCH_CHECK(tiles->dim() == 2 && tiles->size(1) == 3 && max_tile_queries <= 16, "sink_attention: tiles");
+    TORCH_CHECK(tiles->dim() == 2 && tiles->size(1) == 3 && max_tile_queries <= 64, "sink_attention: tiles");
     sink_attention_mfma(q, cache, H, G, dk, vd, block_tables, (int)block_size, positions, (float)scale,
                         (float)softcap, sinkp, all_groups, *tiles, part);
   } else {

@@ -1,14 +1,277 @@
+#include "hip/hip_runtime.h"
 // Tiled MFMA form of the sink attention for bf16 prompt portions.
+//
+// One workgroup (4 waves) per (tile of <= 64 consecutive queries of one
+// sequence, query head). Wave w owns queries 16 w .. 16 w + 15 for the whole
+// kernel: their scores, their online softmax and their value sums, so the
+// waves only meet to stage a block of 64 keys: the head's K rows and the V
+// rows (of every kv head when the weights are mixed across heads, of the
+// head's own kv head otherwise) go through LDS once per 64 queries.
+//   scores   MFMA 16x16x32: A = the wave's queries (registers, loaded once),
+//            B = K rows from LDS
+//   softmax  fp32 in the MFMA's result layout; cap and causal mask per score;
+//            row reductions over the 16 lanes of a row; the sink enters the
+//            denominator once, at the end
+//   values   the fp32 weights go through a wave-private LDS tile to the A
+//            layout and are split into two bf16 terms (p = hi + lo, error
+//            <= 2^-17 p), so the weighted sum keeps fp32-grade weights on
+//            bf16 MFMAs; B = V^T from LDS (staged transposed, so a lane's
+//            eight keys of one value column are one 16-byte read)
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 #include "seqmix_common.h"
 
-bool sink_attention_mfma_fits(int dk, int vd, int G, int all_groups) { return false; }
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16v8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+namespace {
+
+#define SAM_KB 64          // keys per block
+#define SAM_QT 64          // queries per tile
+#define SAM_VP 72          // v_lds row pitch (bf16): 64 keys + 8
+#define SAM_PP 68          // p_lds row pitch (floats): 64 keys + 4
+#define SAM_MAX_KSTEPS 8   // dk <= 256
+
+template <int NT>   // 16-column value tiles held by a wave (NV <= 16 NT)
+__global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
+    const bf16_t* __restrict__ q,         // [Tn, H, dk]
+    const bf16_t* __restrict__ cache,     // [rows, G (dk + vd)]
+    const int* __restrict__ block_tables, int max_nb, int block_size,
+    const int* __restrict__ positions, const int* __restrict__ tiles, int H, int G,
+    int dk, int vd, float scale, float softcap, const float* __restrict__ sink,
+    int all_groups, float* __restrict__ part) {   // [Tn, H, NV]
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int ksteps = (dk + 31) / 32;
+  const int KP = ksteps * 32 + 8;                  // k_lds row pitch (bf16)
+  const int NV = all_groups ? G * vd : vd;
+  const int NVp = (NV + 15) / 16 * 16;
+  bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem);                 // [64][KP]
+  bf16_t* v_lds = k_lds + SAM_KB * KP;                             // [NVp][SAM_VP]
+  float* p_all = reinterpret_cast<float*>(v_lds + NVp * SAM_VP);   // [4][16][SAM_PP]
+  int* krow = reinterpret_cast<int*>(p_all + 4 * 16 * SAM_PP);     // [64]
+
+  const int tile = blockIdx.x, hd = blockIdx.y;
+  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
+  const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, lrow = l & 15, lk = l >> 4;
+  const int W = G * (dk + vd);
+  const int grp = hd / (H / G);
+  const int koff = grp * dk;
+  const int voff = G * dk + (all_groups ? 0 : grp * vd);
+  const int p0 = positions[t0];
+  const int plast = p0 + nq - 1;
+  const int nblk = plast / SAM_KB + 1;
+  const int* bt = block_tables + (int64_t)b * max_nb;
+  float* p_lds = p_all + wave * 16 * SAM_PP;
+  const bool active = wave * 16 < nq;              // uniform per wave
+  const int wave_plast = min(plast, p0 + wave * 16 + 15);
+
+  // the wave's queries as A fragments: row lrow, k = ks * 32 + lk * 8 ..
+  bf16v8 qf[SAM_MAX_KSTEPS];
+  {
+    const int qi = wave * 16 + lrow;
+    const bf16_t* qp = q + ((int64_t)(t0 + min(qi, nq - 1)) * H + hd) * dk;
+    #pragma unroll
+    for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
+      #pragma unroll
+      for (int j = 0; j < 8; ++j) qf[ks][j] = (__bf16)0.0f;
+      const int kk = ks * 32 + lk * 8;
+      if (ks < ksteps && qi < nq && kk < dk) qf[ks] = *reinterpret_cast<const bf16v8*>(qp + kk);
+    }
+  }
+  // padding rows of v_lds (value columns NV .. NVp) stay zero
+  for (int i = tid; i < (NVp - NV) * SAM_VP; i += 256) v_lds[NV * SAM_VP + i] = __float2bfloat16(0.f);
+
+  float m[4], lsum[4];
+  f32x4 acc[NT];
+  #pragma unroll
+  for (int r = 0; r < 4; ++r) { m[r] = -INFINITY; lsum[r] = 0.f; }
+  #pragma unroll
+  for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int j0 = kb * SAM_KB;
+    __syncthreads();                               // the previous block's LDS reads are done
+    if (tid < SAM_KB) {
+      const int j = min(j0 + tid, plast);          // keys past the tile's last are masked below
+      krow[tid] = bt[j / block_size] * block_size + j % block_size;
+    }
+    __syncthreads();
+    // K rows: [key][dk], zero beyond dk
+    for (int i = tid; i < SAM_KB * ksteps * 4; i += 256) {
+      const int key = i / (ksteps * 4), c = (i % (ksteps * 4)) * 8;
+      bf16v8 v;
+      if (c < dk) {
+        v = *reinterpret_cast<const bf16v8*>(cache + (int64_t)krow[key] * W + koff + c);
+      } else {
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (__bf16)0.0f;
+      }
+      *reinterpret_cast<bf16v8*>(k_lds + key * KP + c) = v;
+    }
+    // V rows, transposed: v_lds[column][key]
+    for (int i = tid; i < SAM_KB * (NV / 8); i += 256) {
+      const int key = i % SAM_KB, c = (i / SAM_KB) * 8;
+      const bf16v8 v = *reinterpret_cast<const bf16v8*>(cache + (int64_t)krow[key] * W + voff + c);
+      #pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<__bf16*>(v_lds + (c + j) * SAM_VP + key) = v[j];
+    }
+    __syncthreads();
+    if (!active || j0 > wave_plast) continue;      // no query of this wave sees the block
+
+    // scores of the wave's 16 queries against the 64 keys
+    f32x4 s[4];
+    #pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+      s[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+      #pragma unroll
+      for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
+        if (ks < ksteps) {
+          const bf16v8 kf = *reinterpret_cast<const bf16v8*>(
+              k_lds + (ct * 16 + lrow) * KP + ks * 32 + lk * 8);
+          s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, s[ct], 0, 0, 0);
+        }
+      }
+    }
+    // result layout: reg r -> query lk * 4 + r, lane column lrow -> key ct * 16 + lrow
+    float cr[4];
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int qi = wave * 16 + lk * 4 + r;
+      const int prow = (qi < nq) ? p0 + qi : -1;
+      float sv[4];
+      float bm = -INFINITY;
+      #pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        const int j = j0 + ct * 16 + lrow;
+        float x = s[ct][r] * scale;
+        if (softcap > 0.f) x = softcap * tanhf(x / softcap);
+        sv[ct] = (j <= prow) ? x : -INFINITY;
+        bm = fmaxf(bm, sv[ct]);
+      }
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, SM_WAVE));
+      const float mn = fmaxf(m[r], bm);
+      const float c = (mn == -INFINITY) ? 1.0f : expf(m[r] - mn);
+      float ps = 0.f;
+      #pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        const float pv = (sv[ct] == -INFINITY) ? 0.f : expf(sv[ct] - mn);
+        ps += pv;
+        p_lds[(lk * 4 + r) * SAM_PP + ct * 16 + lrow] = pv;
+      }
+      #pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, SM_WAVE);
+      lsum[r] = lsum[r] * c + ps;
+      m[r] = mn;
+      cr[r] = c;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    // weights as A fragments: row lrow, keys ks2 * 32 + lk * 8 ..
+    bf16v8 a_hi[2], a_lo[2];
+    #pragma unroll
+    for (int ks2 = 0; ks2 < 2; ++ks2) {
+      const float4 w0 = *reinterpret_cast<const float4*>(p_lds + lrow * SAM_PP + ks2 * 32 + lk * 8);
+      const float4 w1 = *reinterpret_cast<const float4*>(p_lds + lrow * SAM_PP + ks2 * 32 + lk * 8 + 4);
+      const float pv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      #pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const __bf16 hi = (__bf16)pv[j];
+        a_hi[ks2][j] = hi;
+        a_lo[ks2][j] = (__bf16)(pv[j] - (float)hi);
+      }
+    }
+    #pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (nt * 16 < NV) {
+        f32x4 a = acc[nt];
+        #pragma unroll
+        for (int r = 0; r < 4; ++r) a[r] *= cr[r];
+        #pragma unroll
+        for (int ks2 = 0; ks2 < 2; ++ks2) {
+          const bf16v8 vf = *reinterpret_cast<const bf16v8*>(
+              v_lds + (nt * 16 + lrow) * SAM_VP + ks2 * 32 + lk * 8);
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi[ks2], vf, a, 0, 0, 0);
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo[ks2], vf, a, 0, 0, 0);
+        }
+        acc[nt] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();               // p_lds is rewritten in the next block
+  }
+
+  if (!active) return;
+  #pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int qi = wave * 16 + lk * 4 + r;
+    if (qi >= nq) continue;
+    float M = m[r], L = lsum[r], e = 1.0f;
+    if (sink != nullptr) {
+      const float sk = sink[hd];
+      M = fmaxf(m[r], sk);
+      e = expf(m[r] - M);
+      L = lsum[r] * e + expf(sk - M);
+    }
+    const float f = e / L;
+    float* dst = part + ((int64_t)(t0 + qi) * H + hd) * NV;
+    #pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int col = nt * 16 + lrow;
+      if (col < NV) dst[col] = acc[nt][r] * f;
+    }
+  }
+}
+
+size_t sam_lds_bytes(int dk, int NV) {
+  const int ksteps = (dk + 31) / 32;
+  const int NVp = (NV + 15) / 16 * 16;
+  return (size_t)SAM_KB * (ksteps * 32 + 8) * 2 + (size_t)NVp * SAM_VP * 2 +
+         (size_t)4 * 16 * SAM_PP * 4 + SAM_KB * 4;
+}
+
+}  // namespace
+
+bool sink_attention_mfma_fits(int dk, int vd, int G, int all_groups) {
+  const int NV = all_groups ? G * vd : vd;
+  return dk % 8 == 0 && vd % 8 == 0 && dk <= 32 * SAM_MAX_KSTEPS && NV <= 768 &&
+         sam_lds_bytes(dk, NV) <= 150 * 1024;
+}
 
 torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, int G, int dk, int vd,
                                   torch::Tensor block_tables, int block_size, torch::Tensor positions,
                                   float scale, float softcap, const float* sink, int all_groups,
                                   torch::Tensor tiles, torch::Tensor part) {
-  TORCH_CHECK(false, "sink_attention_mfma: not available");
+  const int NV = all_groups ? G * vd : vd;
+  TORCH_CHECK(sink_attention_mfma_fits(dk, vd, G, all_groups), "sink_attention_mfma: sizes");
+  const int ntiles = tiles.size(0);
+  if (ntiles == 0) return part;
+  const size_t lds = sam_lds_bytes(dk, NV);
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+#define SAM_LAUNCH(N)                                                                      \
+  do {                                                                                     \
+    auto kern = sink_attention_mfma_kernel<N>;                                             \
+    static int raised = 0;     /* per variant; not repeated under graph capture */         \
+    if (lds > 64 * 1024 && (int)lds > raised) {                                            \
+      TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                 \
+                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, \
+                  "sink attention: cannot raise the LDS limit");                           \
+      raised = (int)lds;                                                                   \
+    }                                                                                      \
+   hipLaunchKernelGGL(( kern), dim3(dim3(ntiles, H)), dim3(256), lds, stream,                                            \
+        reinterpret_cast<const bf16_t*>(q.data_ptr()),                                     \
+        reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),   \
+        (int)block_tables.size(1), block_size, positions.data_ptr<int>(),                  \
+        tiles.data_ptr<int>(), H, G, dk, vd, scale, softcap, sink, all_groups,             \
+        part.data_ptr<float>());                                                           \
+  } while (0)
+  const int nt = (NV + 15) / 16;
+  if (nt <= 4) SAM_LAUNCH(4);
+  else if (nt <= 8) SAM_LAUNCH(8);
+  else if (nt <= 16) SAM_LAUNCH(16);
+  else if (nt <= 32) SAM_LAUNCH(32);
+  else SAM_LAUNCH(48);
+#undef SAM_LAUNCH
+  SM_CHECK_LAUNCH();
   return part;
 }

@@ -57,16 +57,17 @@ def latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
 
 
 QUERY_TILE = 16   # most queries of one sequence the tiled kernel takes at once
+WIDE_QUERY_TILE = 64   # the same for the K/V attention kernel (four waves x 16)
 
 
-def query_tiles(row_lengths):
-    """Cut each batch row's tokens into tiles of up to QUERY_TILE
-    consecutive queries: [(batch row, first flat token, queries)], and the
-    largest tile."""
+def query_tiles(row_lengths, tile=QUERY_TILE):
+    """Cut each batch row's tokens into tiles of up to ``tile`` consecutive
+    queries: [(batch row, first flat token, queries)], and the largest
+    tile."""
     tiles, at = [], 0
     for b, n in enumerate(row_lengths):
-        for k in range(0, n, QUERY_TILE):
-            tiles.append((b, at + k, min(QUERY_TILE, n - k)))
+        for k in range(0, n, tile):
+            tiles.append((b, at + k, min(tile, n - k)))
         at += n
     return tiles, max((t[2] for t in tiles), default=1)
 
@@ -175,9 +176,9 @@ def rope_kv_write(proj, heads, kv_heads, dim, vdim, positions, rope_base,
 def sink_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
                    block_size, cu, tok_seq, positions, scale, softcap, sink,
                    talk, out_dtype, tiles=None, max_tile=0):
-    """``tiles`` (from :func:`query_tiles`) selects the tiled MFMA kernel
-    for bf16 prompt portions; decode steps and fp32 models run one wave per
-    (token, head)."""
+    """``tiles`` (from :func:`query_tiles` with ``WIDE_QUERY_TILE``) selects
+    the tiled MFMA kernel for bf16 prompt portions; decode steps and fp32
+    models run one wave per (token, head)."""
     if q.is_cuda:
         return _ext("sink_attention").sink_attention(
             q, cache, heads, kv_heads, dim, vdim, block_tables, block_size,

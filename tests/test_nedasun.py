@@ -33,7 +33,10 @@ def dev(request):
 
 
 def tol(dtype):
-    return 2e-4 if dtype == torch.float32 else 6e-2
+    # bf16 is a coarse check here: seven layers only 16 wide, and a router
+    # choice may flip on a rounding. The same kernels are held to 2e-4 in
+    # fp32, and the bf16-only tiled attention kernel has a test of its own.
+    return 2e-4 if dtype == torch.float32 else 0.15
 
 
 def rel_err(got, want):
@@ -159,7 +162,7 @@ def _attend(dev, H, G, dk, vd, bs, table, pos, cache, q, scale=1.0, softcap=0.0,
     for b, (_, cnt) in enumerate(rows):
         cu.append(cu[-1] + cnt)
         seq += [b] * cnt
-    tiles, mt = SM.query_tiles([c for _, c in rows])
+    tiles, mt = SM.query_tiles([c for _, c in rows], SM.WIDE_QUERY_TILE)
     return SM.sink_attention(
         q.to(dtype).to(device), cache, H, G, dk, vd, ints(table, device), bs, ints(cu, device),
         ints(seq, device), ints(pos, device), scale, softcap,
@@ -405,6 +408,9 @@ def test_mixed_batch_equals_alone_with_reuse(dev):
     assert not live
     for i in reqs:
         assert rel_err(torch.cat(got[i]), want[i]) < tol(dev[1]), i
+        # what else is in the batch changes nothing beyond rounding
+        alone = run_portions(eng, reqs[i], [len(reqs[i])])
+        assert rel_err(torch.cat(got[i]), alone) < (1e-5 if dev[1] == torch.float32 else 3e-2), i
     assert eng.pool.allocator.num_free == 14 and eng.slots.num_free == 3
 
 
@@ -547,7 +553,7 @@ def test_tiled_attention_kernel_against_plain_op(H, G, dk, vd, lens, talk):
         cu.append(cu[-1] + n)
     sink = torch.randn(H, generator=g).to(device)
     tk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).to(device) if talk else None
-    tiles, mt = SM.query_tiles(lens)
+    tiles, mt = SM.query_tiles(lens, SM.WIDE_QUERY_TILE)
     args = (H, G, dk, vd, ints(tables, device), bs, ints(cu, device), ints(seq, device),
             ints(pos, device), dk ** -0.5, 4.0, sink, tk)
     got = SM.sink_attention(q, cache, *args, torch.bfloat16, tiles=ints(tiles, device).view(-1, 3),
