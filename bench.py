@@ -51,10 +51,12 @@ def parse_args():
                         "no-EOS rounds). Measures in-wave retirement.")
     p.add_argument("--hybrid-bench", type=str, default="",
                    help="instead of the RL round: prefill/decode tokens/s of "
-                        "the Nibalix design beside the dense model of equal "
-                        "size, at these comma-separated sizes (1k,2k)")
+                        "the layer-list designs (Nedasun, Nibalix) beside the "
+                        "dense model of equal size, at these comma-separated "
+                        "sizes (1k,2k)")
     p.add_argument("--hybrid-only", type=str, default="",
-                   help="with --hybrid-bench: run only 'nibalix' or 'dense'")
+                   help="with --hybrid-bench: run only these of 'nedasun', "
+                        "'nibalix', 'dense' (comma-separated)")
     p.add_argument("--tiny", action="store_true",
                    help="tiny model + short generations (debug only; NOT the "
                         "headline config)")
@@ -67,7 +69,8 @@ def main():
         from distrl_llm_amd import bench_hybrid
         dev = torch.device("cuda:0" if torch.cuda.is_available() and not args.cpu
                            else "cpu")
-        which = (args.hybrid_only,) if args.hybrid_only else ("nibalix", "dense")
+        which = (tuple(args.hybrid_only.split(",")) if args.hybrid_only
+                 else ("nedasun", "nibalix", "dense"))
         bench_hybrid.run(args.hybrid_bench.split(","), dev, which=which)
         return
     rank = int(os.environ.get("RANK", "0"))

@@ -1,7 +1,8 @@
-"""Prefill and decode throughput of the Nibalix design beside the dense
-transformer of equal size (``bench.py --hybrid-bench``).
+"""Prefill and decode throughput of the layer-list designs (Nibalix,
+Nedasun) beside one another and beside the dense transformer of equal size
+(``bench.py --hybrid-bench``).
 
-Both models get random weights at layer sizes that resemble a real model
+All models get random weights at layer sizes that resemble a real model
 and run through their own engine's ``generate`` — scheduler, cache, step
 function and sampler included. Prefill tokens/s is timed with one output
 token per prompt; decode tokens/s from the extra time of a longer
@@ -50,11 +51,40 @@ def nibalix_bench_config(s: dict) -> dict:
             "width": s["width"]}
 
 
-def _build_hybrid(s, device, max_len, batch):
+def nedasun_bench_config(s: dict) -> dict:
+    """Same width, depth, head count and expert sizes as the Nibalix config
+    of the size: attention and delta-rule layers alternate (every fourth
+    layer pair starts with a dense feed-forward), 4 query heads per kv
+    head, one identity expert and a shared expert as wide as one expert."""
+    kvh = max(1, s["heads"] // 4)
+    moe = {"kind": "moe", "expert": {"ff": s["ff"], "limit": 7.0},
+           "router": {"experts": s["experts"], "identity": 1, "scale": 1.0,
+                      "top": s["top"]},
+           "shared": {"ff": s["ff"], "limit": 7.0}}
+    dense = {"kind": "dense", "ff": s["top"] * s["ff"], "limit": 7.0}
+    layers = []
+    for i in range(s["layers"]):
+        mlp = dense if i == 0 else moe
+        if i % 2 == 0:
+            mc = {"heads": s["heads"], "kv_heads": kvh, "dim": 128, "vdim": 128,
+                  "scale": 128 ** -0.5, "softcap": 30.0, "v_mix": True,
+                  "rot": {"base": 10000.0, "dims": 64}}
+            layers.append({"type": "attention", "mixer": mc, "mlp": mlp})
+        else:
+            mc = {"heads": s["heads"], "kv_heads": kvh, "dim": 128, "vdim": 128,
+                  "conv": 4}
+            layers.append({"type": "delta", "mixer": mc, "mlp": mlp})
+    return {"architecture": "Nedasun", "layers": layers, "norm": {"eps": 1e-5},
+            "vocab": s["vocab"], "width": s["width"]}
+
+
+def _build_hybrid(s, device, max_len, batch, design="nibalix"):
     from .engine.hybrid_engine import HybridEngine
-    from .models.hybrid import HybridLM, nibalix_spec_from_config
-    model = HybridLM(nibalix_spec_from_config(nibalix_bench_config(s)),
-                     dtype=torch.bfloat16, device=device).random_init(1)
+    from .models.hybrid import (HybridLM, nedasun_spec_from_config,
+                                nibalix_spec_from_config)
+    spec = (nedasun_spec_from_config(nedasun_bench_config(s)) if design == "nedasun"
+            else nibalix_spec_from_config(nibalix_bench_config(s)))
+    model = HybridLM(spec, dtype=torch.bfloat16, device=device).random_init(1)
     cfg = EngineConfig(max_seq_length=max_len, kv_block_size=16,
                        num_kv_blocks=batch * ((max_len + 15) // 16) + 8,
                        num_state_slots=batch, max_num_seqs=batch,
@@ -100,14 +130,16 @@ def measure(engine, vocab, batch, prompt_len, new_tokens, device):
             "prefill_s": t_pre, "decode_ms_per_step": 1e3 * dec / (new_tokens - 1)}
 
 
-def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("nibalix", "dense")):
+def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("nedasun", "nibalix", "dense")):
     out = []
     for name in sizes:
         s = SIZES[name]
         max_len = prompt_len + new_tokens + 1
         for kind in which:
-            eng = (_build_hybrid if kind == "nibalix" else _build_dense)(
-                s, device, max_len, batch)
+            if kind == "dense":
+                eng = _build_dense(s, device, max_len, batch)
+            else:
+                eng = _build_hybrid(s, device, max_len, batch, design=kind)
             r = measure(eng, s["vocab"], batch, prompt_len, new_tokens, device)
             line = {"bench": "hybrid", "size": name, "model": kind, "batch": batch,
                     "prompt_len": prompt_len, "new_tokens": new_tokens, "dtype": "bf16",

@@ -222,6 +222,11 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
                                   float scale, float softcap, const float* sink, int all_groups,
                                   torch::Tensor tiles, torch::Tensor part);
 bool sink_attention_mfma_fits(int dk, int vd, int G, int all_groups);
+torch::Tensor sink_attention_heads(torch::Tensor q, torch::Tensor cache, int H, int G, int dk, int vd,
+                                   torch::Tensor block_tables, int block_size, torch::Tensor tok_seq,
+                                   torch::Tensor positions, float scale, float softcap,
+                                   const float* sink, int all_groups, torch::Tensor part);
+bool sink_attention_heads_fits(int H, int dk, int vd, int G);
 
 torch::Tensor sink_attention(torch::Tensor q, torch::Tensor cache, int64_t heads,
                              int64_t kv_heads, int64_t dim, int64_t vdim,
@@ -266,6 +271,11 @@ torch::Tensor sink_attention(torch::Tensor q, torch::Tensor cache, int64_t heads
     TORCH_CHECK(tiles->dim() == 2 && tiles->size(1) == 3 && max_tile_queries <= 64, "sink_attention: tiles");
     sink_attention_mfma(q, cache, H, G, dk, vd, block_tables, (int)block_size, positions, (float)scale,
                         (float)softcap, sinkp, all_groups, *tiles, part);
+  } else if (bf16 && tiles.has_value() && max_tile_queries == 1 &&
+             sink_attention_heads_fits(H, dk, vd, G)) {
+    // a decode step: one token per row
+    sink_attention_heads(q, cache, H, G, dk, vd, block_tables, (int)block_size, tok_seq, positions,
+                         (float)scale, (float)softcap, sinkp, all_groups, part);
   } else {
     const size_t lds = (dk + 64) * sizeof(float) + 64 * sizeof(int);
     dim3 grid(Tn, H);

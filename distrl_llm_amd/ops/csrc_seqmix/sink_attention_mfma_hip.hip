@@ -1,5 +1,7 @@
 #include "hip/hip_runtime.h"
-// Tiled MFMA form of the sink attention for bf16 prompt portions.
+// Tiled MFMA forms of the sink attention for bf16: prompt portions (a tile =
+// up to 64 queries of one head) and decode steps (HEADS: a tile = the heads
+// of one token, the key range split over workgroups and merged afterwards).
 //
 // One workgroup (4 waves) per (tile of <= 64 consecutive queries of one
 // sequence, query head). Wave w owns queries 16 w .. 16 w + 15 for the whole
@@ -17,6 +19,11 @@
 //            <= 2^-17 p), so the weighted sum keeps fp32-grade weights on
 //            bf16 MFMAs; B = V^T from LDS (staged transposed, so a lane's
 //            eight keys of one value column are one 16-byte read)
+// HEADS: wave w owns heads 16 w .. 16 w + 15 of one decoded token. Their kv
+// heads differ, so the scores are taken per kv head (B = K rows straight from
+// the cache: every K element feeds one MFMA only) and each row keeps the tile
+// of its own kv head; the value sums always run over every kv head and the
+// merge kernel keeps what the head needs.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 #include "seqmix_common.h"
@@ -32,50 +39,62 @@ namespace {
 #define SAM_PP 68          // p_lds row pitch (floats): 64 keys + 4
 #define SAM_MAX_KSTEPS 8   // dk <= 256
 
-template <int NT>   // 16-column value tiles held by a wave (NV <= 16 NT)
+template <int NT, bool HEADS>   // NT: 16-column value tiles held by a wave (NV <= 16 NT)
 __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     const bf16_t* __restrict__ q,         // [Tn, H, dk]
     const bf16_t* __restrict__ cache,     // [rows, G (dk + vd)]
     const int* __restrict__ block_tables, int max_nb, int block_size,
-    const int* __restrict__ positions, const int* __restrict__ tiles, int H, int G,
-    int dk, int vd, float scale, float softcap, const float* __restrict__ sink,
-    int all_groups, float* __restrict__ part) {   // [Tn, H, NV]
+    const int* __restrict__ positions,
+    const int* __restrict__ tiles,        // query tiles, or tok_seq when HEADS
+    int H, int G, int dk, int vd, float scale, float softcap,
+    const float* __restrict__ sink, int all_groups,
+    float* __restrict__ part,             // [Tn, H, NV]; HEADS: [Tn, H, ksplit, NV] unnormalised
+    int ksplit, float* __restrict__ part_ml) {     // HEADS: [Tn, H, ksplit, 2] = (max, sum)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int ksteps = (dk + 31) / 32;
-  const int KP = ksteps * 32 + 8;                  // k_lds row pitch (bf16)
-  const int NV = all_groups ? G * vd : vd;
+  const int KP = HEADS ? 0 : ksteps * 32 + 8;      // k_lds row pitch (bf16)
+  const int NV = (HEADS || all_groups) ? G * vd : vd;
   const int NVp = (NV + 15) / 16 * 16;
   bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem);                 // [64][KP]
   bf16_t* v_lds = k_lds + SAM_KB * KP;                             // [NVp][SAM_VP]
   float* p_all = reinterpret_cast<float*>(v_lds + NVp * SAM_VP);   // [4][16][SAM_PP]
   int* krow = reinterpret_cast<int*>(p_all + 4 * 16 * SAM_PP);     // [64]
 
-  const int tile = blockIdx.x, hd = blockIdx.y;
-  const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
+  const int tile = blockIdx.x;
+  const int hd = HEADS ? 0 : blockIdx.y;
+  const int b = HEADS ? tiles[tile] : tiles[3 * tile];
+  const int t0 = HEADS ? tile : tiles[3 * tile + 1];
+  const int nq = HEADS ? 1 : tiles[3 * tile + 2];
   const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, lrow = l & 15, lk = l >> 4;
   const int W = G * (dk + vd);
-  const int grp = hd / (H / G);
+  const int rep = H / G;
+  const int grp = hd / rep;
   const int koff = grp * dk;
-  const int voff = G * dk + (all_groups ? 0 : grp * vd);
+  const int voff = G * dk + ((HEADS || all_groups) ? 0 : grp * vd);
   const int p0 = positions[t0];
   const int plast = p0 + nq - 1;
   const int nblk = plast / SAM_KB + 1;
   const int* bt = block_tables + (int64_t)b * max_nb;
   float* p_lds = p_all + wave * 16 * SAM_PP;
-  const bool active = wave * 16 < nq;              // uniform per wave
-  const int wave_plast = min(plast, p0 + wave * 16 + 15);
+  // uniform per wave: it has rows (queries of the tile, or heads of the token)
+  const bool active = HEADS ? (wave * 16 < H) : (wave * 16 < nq);
+  const int wave_plast = HEADS ? plast : min(plast, p0 + wave * 16 + 15);
+  const int kb_lo = HEADS ? (int)(((int64_t)nblk * blockIdx.y) / ksplit) : 0;
+  const int kb_hi = HEADS ? (int)(((int64_t)nblk * (blockIdx.y + 1)) / ksplit) : nblk;
 
-  // the wave's queries as A fragments: row lrow, k = ks * 32 + lk * 8 ..
+  // the wave's rows as A fragments: row lrow, k = ks * 32 + lk * 8 ..
   bf16v8 qf[SAM_MAX_KSTEPS];
   {
     const int qi = wave * 16 + lrow;
-    const bf16_t* qp = q + ((int64_t)(t0 + min(qi, nq - 1)) * H + hd) * dk;
+    const bool row_ok = HEADS ? (qi < H) : (qi < nq);
+    const bf16_t* qp = HEADS ? q + ((int64_t)t0 * H + min(qi, H - 1)) * dk
+                             : q + ((int64_t)(t0 + min(qi, nq - 1)) * H + hd) * dk;
     #pragma unroll
     for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
       #pragma unroll
       for (int j = 0; j < 8; ++j) qf[ks][j] = (__bf16)0.0f;
       const int kk = ks * 32 + lk * 8;
-      if (ks < ksteps && qi < nq && kk < dk) qf[ks] = *reinterpret_cast<const bf16v8*>(qp + kk);
+      if (ks < ksteps && row_ok && kk < dk) qf[ks] = *reinterpret_cast<const bf16v8*>(qp + kk);
     }
   }
   // padding rows of v_lds (value columns NV .. NVp) stay zero
@@ -88,7 +107,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
   #pragma unroll
   for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = 0; kb < nblk; ++kb) {
+  for (int kb = kb_lo; kb < kb_hi; ++kb) {
     const int j0 = kb * SAM_KB;
     __syncthreads();                               // the previous block's LDS reads are done
     if (tid < SAM_KB) {
@@ -97,7 +116,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     }
     __syncthreads();
     // K rows: [key][dk], zero beyond dk
-    for (int i = tid; i < SAM_KB * ksteps * 4; i += 256) {
+    if (!HEADS) for (int i = tid; i < SAM_KB * ksteps * 4; i += 256) {
       const int key = i / (ksteps * 4), c = (i % (ksteps * 4)) * 8;
       bf16v8 v;
       if (c < dk) {
@@ -119,17 +138,42 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     __syncthreads();
     if (!active || j0 > wave_plast) continue;      // no query of this wave sees the block
 
-    // scores of the wave's 16 queries against the 64 keys
+    // scores of the wave's 16 rows against the 64 keys
     f32x4 s[4];
     #pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
-      s[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int ct = 0; ct < 4; ++ct) s[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (HEADS) {
+      const int c_hi = min(G - 1, (wave * 16 + 15) / rep);
+      for (int c = (wave * 16) / rep; c <= c_hi; ++c) {
+        #pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+          const bf16_t* kp = cache + (int64_t)krow[ct * 16 + lrow] * W + c * dk + lk * 8;
+          #pragma unroll
+          for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
+            if (ks < ksteps) {
+              bf16v8 kf;
+              #pragma unroll
+              for (int j = 0; j < 8; ++j) kf[j] = (__bf16)0.0f;
+              if (ks * 32 + lk * 8 < dk) kf = *reinterpret_cast<const bf16v8*>(kp + ks * 32);
+              sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, sc, 0, 0, 0);
+            }
+          }
+          #pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if ((wave * 16 + lk * 4 + r) / rep == c) s[ct][r] = sc[r];
+        }
+      }
+    } else {
       #pragma unroll
-      for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
-        if (ks < ksteps) {
-          const bf16v8 kf = *reinterpret_cast<const bf16v8*>(
-              k_lds + (ct * 16 + lrow) * KP + ks * 32 + lk * 8);
-          s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, s[ct], 0, 0, 0);
+      for (int ct = 0; ct < 4; ++ct) {
+        #pragma unroll
+        for (int ks = 0; ks < SAM_MAX_KSTEPS; ++ks) {
+          if (ks < ksteps) {
+            const bf16v8 kf = *reinterpret_cast<const bf16v8*>(
+                k_lds + (ct * 16 + lrow) * KP + ks * 32 + lk * 8);
+            s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, s[ct], 0, 0, 0);
+          }
         }
       }
     }
@@ -138,7 +182,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int qi = wave * 16 + lk * 4 + r;
-      const int prow = (qi < nq) ? p0 + qi : -1;
+      const int prow = HEADS ? ((qi < H) ? p0 : -1) : ((qi < nq) ? p0 + qi : -1);
       float sv[4];
       float bm = -INFINITY;
       #pragma unroll
@@ -202,6 +246,25 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
   }
 
   if (!active) return;
+  if (HEADS) {
+    // unnormalised partial of this key range; the merge kernel adds the sink
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int head = wave * 16 + lk * 4 + r;
+      if (head >= H) continue;
+      const int64_t o = ((int64_t)t0 * H + head) * ksplit + blockIdx.y;
+      if (lrow == 0) {
+        part_ml[o * 2] = m[r];
+        part_ml[o * 2 + 1] = lsum[r];
+      }
+      #pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int col = nt * 16 + lrow;
+        if (col < NV) part[o * NV + col] = acc[nt][r];
+      }
+    }
+    return;
+  }
   #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int qi = wave * 16 + lk * 4 + r;
@@ -223,10 +286,38 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
   }
 }
 
-size_t sam_lds_bytes(int dk, int NV) {
+// Merge the key ranges of one (token, head): M = max(m_s, sink),
+// L = sum_s l_s e^(m_s - M) + e^(sink - M), out = sum_s acc_s e^(m_s - M) / L,
+// over every kv head's columns (all_groups) or the head's own.
+__global__ __launch_bounds__(256) void sink_attention_merge_kernel(
+    const float* __restrict__ pacc, const float* __restrict__ pml,
+    const float* __restrict__ sink, int H, int G, int vd, int ksplit, int all_groups,
+    float* __restrict__ part) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int NVin = G * vd;
+  const int NVout = all_groups ? NVin : vd;
+  const int c0 = all_groups ? 0 : (h / (H / G)) * vd;
+  const float* ml = pml + ((t * H + h) * ksplit) * 2;
+  float M = (sink != nullptr) ? sink[h] : -INFINITY;
+  for (int s = 0; s < ksplit; ++s) M = fmaxf(M, ml[2 * s]);
+  float L = (sink != nullptr) ? expf(sink[h] - M) : 0.f;
+  for (int s = 0; s < ksplit; ++s)
+    if (ml[2 * s] != -INFINITY) L += ml[2 * s + 1] * expf(ml[2 * s] - M);
+  const float inv = 1.0f / L;
+  for (int col = threadIdx.x; col < NVout; col += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < ksplit; ++s)
+      if (ml[2 * s] != -INFINITY)
+        a += pacc[((t * H + h) * ksplit + s) * NVin + c0 + col] * expf(ml[2 * s] - M);
+    part[(t * H + h) * NVout + col] = a * inv;
+  }
+}
+
+size_t sam_lds_bytes(int dk, int NV, bool heads) {
   const int ksteps = (dk + 31) / 32;
   const int NVp = (NV + 15) / 16 * 16;
-  return (size_t)SAM_KB * (ksteps * 32 + 8) * 2 + (size_t)NVp * SAM_VP * 2 +
+  return (heads ? 0 : (size_t)SAM_KB * (ksteps * 32 + 8) * 2) + (size_t)NVp * SAM_VP * 2 +
          (size_t)4 * 16 * SAM_PP * 4 + SAM_KB * 4;
 }
 
@@ -235,7 +326,12 @@ size_t sam_lds_bytes(int dk, int NV) {
 bool sink_attention_mfma_fits(int dk, int vd, int G, int all_groups) {
   const int NV = all_groups ? G * vd : vd;
   return dk % 8 == 0 && vd % 8 == 0 && dk <= 32 * SAM_MAX_KSTEPS && NV <= 768 &&
-         sam_lds_bytes(dk, NV) <= 150 * 1024;
+         sam_lds_bytes(dk, NV, false) <= 150 * 1024;
+}
+
+bool sink_attention_heads_fits(int H, int dk, int vd, int G) {
+  return dk % 8 == 0 && vd % 8 == 0 && dk <= 32 * SAM_MAX_KSTEPS && G * vd <= 768 && H <= 64 &&
+         sam_lds_bytes(dk, G * vd, true) <= 150 * 1024;
 }
 
 torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, int G, int dk, int vd,
@@ -246,11 +342,11 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
   TORCH_CHECK(sink_attention_mfma_fits(dk, vd, G, all_groups), "sink_attention_mfma: sizes");
   const int ntiles = tiles.size(0);
   if (ntiles == 0) return part;
-  const size_t lds = sam_lds_bytes(dk, NV);
+  const size_t lds = sam_lds_bytes(dk, NV, false);
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
 #define SAM_LAUNCH(N)                                                                      \
   do {                                                                                     \
-    auto kern = sink_attention_mfma_kernel<N>;                                             \
+    auto kern = sink_attention_mfma_kernel<N, false>;                                           \
     static int raised = 0;     /* per variant; not repeated under graph capture */         \
     if (lds > 64 * 1024 && (int)lds > raised) {                                            \
       TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                 \
@@ -263,7 +359,7 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
         reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),   \
         (int)block_tables.size(1), block_size, positions.data_ptr<int>(),                  \
         tiles.data_ptr<int>(), H, G, dk, vd, scale, softcap, sink, all_groups,             \
-        part.data_ptr<float>());                                                           \
+        part.data_ptr<float>(), 1, nullptr);                                               \
   } while (0)
   const int nt = (NV + 15) / 16;
   if (nt <= 4) SAM_LAUNCH(4);
@@ -272,6 +368,57 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
   else if (nt <= 32) SAM_LAUNCH(32);
   else SAM_LAUNCH(48);
 #undef SAM_LAUNCH
+  SM_CHECK_LAUNCH();
+  return part;
+}
+
+// Decode steps: every row of the step is one token. The key range of a token
+// is split over ksplit workgroups, chosen from host-side sizes only (token
+// count, block-table width) so that a captured step keeps its grid.
+torch::Tensor sink_attention_heads(torch::Tensor q, torch::Tensor cache, int H, int G, int dk, int vd,
+                                   torch::Tensor block_tables, int block_size, torch::Tensor tok_seq,
+                                   torch::Tensor positions, float scale, float softcap,
+                                   const float* sink, int all_groups, torch::Tensor part) {
+  TORCH_CHECK(sink_attention_heads_fits(H, dk, vd, G), "sink_attention_heads: sizes");
+  const int64_t Tn = q.size(0);
+  if (Tn == 0) return part;
+  const int NV = G * vd;
+  const int64_t max_keys = block_tables.size(1) * (int64_t)block_size;
+  const int max_blk = (int)std::max<int64_t>(1, SM_CDIV(max_keys, SAM_KB));
+  const int ksplit = (int)std::min<int64_t>(max_blk, std::max<int64_t>(1, 1024 / Tn));
+  auto f32 = q.options().dtype(at::kFloat);
+  auto pacc = torch::empty({Tn, H, ksplit, NV}, f32);
+  auto pml = torch::empty({Tn, H, ksplit, 2}, f32);
+  const size_t lds = sam_lds_bytes(dk, NV, true);
+  auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+#define SAM_LAUNCH(N)                                                                      \
+  do {                                                                                     \
+    auto kern = sink_attention_mfma_kernel<N, true>;                                       \
+    static int raised = 0;                                                                 \
+    if (lds > 64 * 1024 && (int)lds > raised) {                                            \
+      TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                 \
+                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, \
+                  "sink attention: cannot raise the LDS limit");                           \
+      raised = (int)lds;                                                                   \
+    }                                                                                      \
+   hipLaunchKernelGGL(( kern), dim3(dim3(Tn, ksplit)), dim3(256), lds, stream,                                           \
+        reinterpret_cast<const bf16_t*>(q.data_ptr()),                                     \
+        reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),   \
+        (int)block_tables.size(1), block_size, positions.data_ptr<int>(),                  \
+        tok_seq.data_ptr<int>(), H, G, dk, vd, scale, softcap, sink, all_groups,           \
+        pacc.data_ptr<float>(), ksplit, pml.data_ptr<float>());                            \
+  } while (0)
+  const int nt = (NV + 15) / 16;
+  if (nt <= 4) SAM_LAUNCH(4);
+  else if (nt <= 8) SAM_LAUNCH(8);
+  else if (nt <= 16) SAM_LAUNCH(16);
+  else if (nt <= 32) SAM_LAUNCH(32);
+  else SAM_LAUNCH(48);
+#undef SAM_LAUNCH
+  SM_CHECK_LAUNCH();
+ hipLaunchKernelGGL(( sink_attention_merge_kernel), dim3(dim3(Tn, H)), dim3(256), 0, stream, 
+      pacc.data_ptr<float>(), pml.data_ptr<float>(), sink, H, G, vd, ksplit, all_groups,
+      part.data_ptr<float>());
   SM_CHECK_LAUNCH();
   return part;
 }

@@ -529,14 +529,19 @@ def test_captured_decode_equals_eager():
 @pytest.mark.parametrize("H,G,dk,vd,lens,talk", [(4, 2, 64, 48, [300, 1, 37, 2], True),
                                                  (6, 3, 128, 128, [70, 16, 17], True),
                                                  (4, 4, 32, 64, [129, 5], False),
-                                                 (2, 1, 96, 40, [65, 33], True)])
+                                                 (2, 1, 96, 40, [65, 33], True),
+                                                 (8, 2, 128, 64, [1, 1, 1, 1], True),
+                                                 (4, 4, 32, 64, [1, 1, 1], False),
+                                                 (48, 8, 64, 32, [1, 1], True),
+                                                 (6, 3, 40, 24, [1, 1, 1, 1], True)])
 def test_tiled_attention_kernel_against_plain_op(H, G, dk, vd, lens, talk):
-    """bf16 prompt portions take the tiled MFMA kernel; the fp32 reference
-    op on the same cache rows must agree. Rows start at uneven positions
-    inside their sequences and pages are scattered."""
+    """bf16 prompt portions take the tiled MFMA kernel, steps of single
+    tokens its heads-of-one-token form with split key ranges; the fp32
+    reference op on the same cache rows must agree. Rows start at uneven
+    positions inside their sequences and pages are scattered."""
     device, bs = torch.device("cuda"), 16
     g = torch.Generator().manual_seed(8)
-    starts = [5, 40, 0, 130][:len(lens)]
+    starts = [5, 40, 0, 330][:len(lens)]
     nb = [(s + n + bs - 1) // bs for s, n in zip(starts, lens)]
     perm = torch.randperm(sum(nb) + 2, generator=g).tolist()
     tables, at = [], 0
