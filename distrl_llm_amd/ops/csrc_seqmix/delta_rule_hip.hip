@@ -6,7 +6,8 @@
 //                   decay = exp(-exp(a_log) softplus(a + dt_bias)), all fp32
 //   delta_scan      per (sequence row, head, block of value columns): walks
 //                   the row's tokens in order with the state in registers,
-//                   S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
+//                   S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
+//                   inputs arrive in chunks through LDS, one chunk ahead
 //   delta_finish    per (token, head): o / rms(o) * norm_w * silu(gate)
 // The scan is strictly sequential over a row's tokens, so a prompt cut into
 // portions gives bit-identical states and outputs.
@@ -54,15 +55,25 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
 
 // One wave per (row, head, 64 / KS value columns). Lane = (column, ks): it
 // holds rows ks * 32 .. ks * 32 + 31 of its column; dot products over the key
-// axis are finished with shuffles over the KS lanes of a column.
+// axis are finished with shuffles over the KS lanes of a column. The walk is
+// latency-bound, so the tokens come in chunks of DR_CH: a chunk's unit q/k
+// rows, decays and strengths sit in LDS (every lane reads the same few
+// addresses), the lane's own v entries in registers, and the next chunk is
+// fetched into registers while the current one is walked.
+#define DR_CH 16
 template <typename T, int KS>
 __global__ __launch_bounds__(64) void delta_scan_kernel(
     const T* __restrict__ qkv, int C, const float* __restrict__ qn,
     const float* __restrict__ kn, const float* __restrict__ beta,
     const float* __restrict__ decay, float* __restrict__ state,
     const int* __restrict__ cu, const int* __restrict__ slots, int H, int G, int dk,
-    int dkp, int vd, float* __restrict__ o) {
+    int vd, float* __restrict__ o) {
   constexpr int COLS = 64 / KS;
+  constexpr int DKP = KS * DR_ROWS;
+  constexpr int ROW4 = DKP / 4;                 // float4 per q or k row
+  constexpr int NPRE = DR_CH * 2 * ROW4 / 64;   // float4 per lane and chunk
+  __shared__ float4 kq4[DR_CH * 2 * ROW4];      // [token][k | q][DKP]
+  __shared__ float sc[DR_CH * 2];               // [token][decay | beta]
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
   const int ks = lane % KS;
@@ -80,37 +91,88 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
     S[r] = (live && k < dk) ? Sp[(int64_t)k * vd] : 0.f;
   }
   const int voff = 2 * G * dk + h * vd + (live ? col : 0);
-  for (int t = t0; t < t1; ++t) {
-    const float* kp = kn + ((int64_t)t * G + g) * dkp + ks * DR_ROWS;
-    const float* qp = qn + ((int64_t)t * G + g) * dkp + ks * DR_ROWS;
-    const float dec = decay[(int64_t)t * H + h], bt = beta[(int64_t)t * H + h];
-    const float v = to_f(qkv[(int64_t)t * C + voff]);
-    float kk[DR_ROWS], qq[DR_ROWS];
+
+  float4 pre[NPRE];
+  float pv[DR_CH], pvn[DR_CH];
+  float psc = 0.f;
+  // fetch a chunk into registers: q/k rows (linear float4 index = LDS index),
+  // the lane's v entries, and decay/beta of token lane / 2
+  auto fetch = [&](int tb, int n, float* vout) {
     #pragma unroll
-    for (int r = 0; r < DR_ROWS; r += 4) {
-      const float4 k4 = *reinterpret_cast<const float4*>(kp + r);
-      const float4 q4 = *reinterpret_cast<const float4*>(qp + r);
-      kk[r] = k4.x; kk[r + 1] = k4.y; kk[r + 2] = k4.z; kk[r + 3] = k4.w;
-      qq[r] = q4.x; qq[r + 1] = q4.y; qq[r + 2] = q4.z; qq[r + 3] = q4.w;
-    }
-    float sk = 0.f;
-    #pragma unroll
-    for (int r = 0; r < DR_ROWS; ++r) {
-      S[r] *= dec;
-      sk = fmaf(S[r], kk[r], sk);
+    for (int j = 0; j < NPRE; ++j) {
+      const int i = lane + 64 * j;
+      const int tok = i / (2 * ROW4), rem = i % (2 * ROW4);
+      const float* src = (rem >= ROW4 ? qn : kn) + ((int64_t)(tb + min(tok, n - 1)) * G + g) * DKP;
+      pre[j] = reinterpret_cast<const float4*>(src)[rem % ROW4];
     }
     #pragma unroll
-    for (int off = 1; off < KS; off <<= 1) sk += __shfl_xor(sk, off, SM_WAVE);
-    const float u = bt * (v - sk);
-    float so = 0.f;
-    #pragma unroll
-    for (int r = 0; r < DR_ROWS; ++r) {
-      S[r] = fmaf(kk[r], u, S[r]);
-      so = fmaf(S[r], qq[r], so);
+    for (int i = 0; i < DR_CH; ++i)
+      vout[i] = to_f(qkv[(int64_t)(tb + min(i, n - 1)) * C + voff]);
+    if (lane < 2 * DR_CH) {
+      const int64_t t = tb + min(lane >> 1, n - 1);
+      psc = (lane & 1) ? beta[t * H + h] : decay[t * H + h];
     }
+  };
+  auto stash = [&]() {
     #pragma unroll
-    for (int off = 1; off < KS; off <<= 1) so += __shfl_xor(so, off, SM_WAVE);
-    if (live && ks == 0) o[((int64_t)t * H + h) * vd + col] = so;
+    for (int j = 0; j < NPRE; ++j) kq4[lane + 64 * j] = pre[j];
+    if (lane < 2 * DR_CH) sc[lane] = psc;
+  };
+
+  fetch(t0, min(DR_CH, t1 - t0), pv);
+  stash();
+  __syncthreads();
+  for (int tb = t0; tb < t1; tb += DR_CH) {
+    const int n = min(DR_CH, t1 - tb);
+    const int nn = min(DR_CH, t1 - tb - DR_CH);
+    if (nn > 0) fetch(tb + DR_CH, nn, pvn);
+    #pragma unroll
+    for (int i = 0; i < DR_CH; ++i) {
+      if (i >= n) break;
+      const float4* kp = kq4 + (i * 2) * ROW4 + ks * (DR_ROWS / 4);
+      const float4* qp = kp + ROW4;
+      const float dec = sc[2 * i], bt = sc[2 * i + 1];
+      // four partial sums per dot product: no 32-long dependent FMA chain
+      float sk0 = 0.f, sk1 = 0.f, sk2 = 0.f, sk3 = 0.f;
+      #pragma unroll
+      for (int r = 0; r < DR_ROWS; r += 4) {
+        const float4 k4 = kp[r / 4];
+        S[r] *= dec; S[r + 1] *= dec; S[r + 2] *= dec; S[r + 3] *= dec;
+        sk0 = fmaf(S[r], k4.x, sk0);
+        sk1 = fmaf(S[r + 1], k4.y, sk1);
+        sk2 = fmaf(S[r + 2], k4.z, sk2);
+        sk3 = fmaf(S[r + 3], k4.w, sk3);
+      }
+      float sk = (sk0 + sk1) + (sk2 + sk3);
+      #pragma unroll
+      for (int off = 1; off < KS; off <<= 1) sk += __shfl_xor(sk, off, SM_WAVE);
+      const float u = bt * (pv[i] - sk);
+      float so0 = 0.f, so1 = 0.f, so2 = 0.f, so3 = 0.f;
+      #pragma unroll
+      for (int r = 0; r < DR_ROWS; r += 4) {
+        const float4 k4 = kp[r / 4];
+        const float4 q4 = qp[r / 4];
+        S[r] = fmaf(k4.x, u, S[r]);
+        S[r + 1] = fmaf(k4.y, u, S[r + 1]);
+        S[r + 2] = fmaf(k4.z, u, S[r + 2]);
+        S[r + 3] = fmaf(k4.w, u, S[r + 3]);
+        so0 = fmaf(S[r], q4.x, so0);
+        so1 = fmaf(S[r + 1], q4.y, so1);
+        so2 = fmaf(S[r + 2], q4.z, so2);
+        so3 = fmaf(S[r + 3], q4.w, so3);
+      }
+      float so = (so0 + so1) + (so2 + so3);
+      #pragma unroll
+      for (int off = 1; off < KS; off <<= 1) so += __shfl_xor(so, off, SM_WAVE);
+      if (live && ks == 0) o[((int64_t)(tb + i) * H + h) * vd + col] = so;
+    }
+    __syncthreads();
+    if (nn > 0) {
+      stash();
+      #pragma unroll
+      for (int i = 0; i < DR_CH; ++i) pv[i] = pvn[i];
+    }
+    __syncthreads();
   }
   #pragma unroll
   for (int r = 0; r < DR_ROWS; ++r) {
@@ -140,11 +202,11 @@ __global__ __launch_bounds__(64) void delta_finish_kernel(
 template <typename T>
 void launch_scan(int KS, dim3 grid, hipStream_t stream, const T* qkv, int C, const float* qn,
                  const float* kn, const float* beta, const float* decay, float* state,
-                 const int* cu, const int* slots, int H, int G, int dk, int dkp, int vd, float* o) {
+                 const int* cu, const int* slots, int H, int G, int dk, int vd, float* o) {
 #define DR_CASE(N)                                                                       \
   case N:                                                                                \
    hipLaunchKernelGGL(( delta_scan_kernel<T, N>), dim3(dim3(grid.x, grid.y, SM_CDIV(vd, 64 / N))), dim3(64), 0, stream,  \
-        qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, dkp, vd, o);            \
+        qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, vd, o);                 \
     break;
   switch (KS) {
     DR_CASE(1) DR_CASE(2) DR_CASE(4) DR_CASE(8)
@@ -198,7 +260,7 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
     SM_CHECK_LAUNCH();
     launch_scan<bf16_t>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                         beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
-                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, dkp, vd, o.data_ptr<float>());
+                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();
    hipLaunchKernelGGL(( delta_finish_kernel<bf16_t>), dim3(gfin), dim3(64), 0, stream, 
         o.data_ptr<float>(), reinterpret_cast<const bf16_t*>(gate.data_ptr()), gate.stride(0),
@@ -211,7 +273,7 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
     SM_CHECK_LAUNCH();
     launch_scan<float>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                        beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
-                       cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, dkp, vd, o.data_ptr<float>());
+                       cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();
    hipLaunchKernelGGL(( delta_finish_kernel<float>), dim3(gfin), dim3(64), 0, stream, 
         o.data_ptr<float>(), gate.data_ptr<float>(), gate.stride(0), onorm_w.data_ptr<float>(),
