@@ -133,9 +133,10 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
       const float dec = sc[2 * i], bt = sc[2 * i + 1];
       // four partial sums per dot product: no 32-long dependent FMA chain
       float sk0 = 0.f, sk1 = 0.f, sk2 = 0.f, sk3 = 0.f;
+      float4 kk[DR_ROWS / 4];             // read once: LDS bandwidth bounds the walk
       #pragma unroll
       for (int r = 0; r < DR_ROWS; r += 4) {
-        const float4 k4 = kp[r / 4];
+        const float4 k4 = kk[r / 4] = kp[r / 4];
         S[r] *= dec; S[r + 1] *= dec; S[r + 2] *= dec; S[r + 3] *= dec;
         sk0 = fmaf(S[r], k4.x, sk0);
         sk1 = fmaf(S[r + 1], k4.y, sk1);
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
       float so0 = 0.f, so1 = 0.f, so2 = 0.f, so3 = 0.f;
       #pragma unroll
       for (int r = 0; r < DR_ROWS; r += 4) {
-        const float4 k4 = kp[r / 4];
+        const float4 k4 = kk[r / 4];
         const float4 q4 = qp[r / 4];
         S[r] = fmaf(k4.x, u, S[r]);
         S[r + 1] = fmaf(k4.y, u, S[r + 1]);
