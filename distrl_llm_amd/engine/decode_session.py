@@ -236,7 +236,7 @@ class CachedDecodeSession(DecodeSession):
 
     Gated off by default (DISTRL_GRAPH_CACHE=1): the padding/reset state
     machine is CPU-tested via DISTRL_FORCE_SESSION; flipping the default
-    needs a GPU validation pass (round-2).
+    needs a GPU validation pass.
     """
 
     def __init__(self, engine, n_pad: int, sp: SamplingParams,

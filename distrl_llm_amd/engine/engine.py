@@ -374,7 +374,7 @@ class Engine:
         """DecodeSession per wave, with cached state buffers + captured
         hipGraph keyed on (padded N, params) reused across waves — saves
         the ~0.2-0.4 s/round re-capture cost (docs/ROADMAP.md #4).
-        GPU-validated round 2: cached-vs-fresh greedy equality
+        GPU-validated: cached-vs-fresh greedy equality
         (tests/test_engine_gpu.py::test_session_cache_vs_fresh_identical)
         and identical fuzz behavior over 15 randomized trials.
         DISTRL_GRAPH_CACHE=0 reverts to per-wave sessions."""

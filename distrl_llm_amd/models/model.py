@@ -214,7 +214,7 @@ class CausalLM(nn.Module):
         OOM'd the 72B dual-role trial)."""
         if keep_bf16 is None:
             # auto: free only when the bf16 image threatens residency
-            # (72B: image 145 GiB; 32B keeps its image — measured round 1
+            # (72B: image 145 GiB; 32B keeps its image — measured
             # at 199 GiB peak with the faster hipBLASLt learner path)
             dev = next(self.parameters()).device
             n_params = sum(p.numel() for p in self.parameters())

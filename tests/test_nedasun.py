@@ -452,6 +452,21 @@ def test_long_prompt_beside_short_rows(dev):
     assert rel_err(out[139:], O.forward(cfg, W, b)[0]) < tol(dev[1])
 
 
+def test_portions_cut_at_kernel_chunk_edges(dev):
+    """The kernels work in chunks of their own (16-token scan chunks, 16-row
+    and 64-query tiles, 64-key blocks, 16-token pages here): portions end
+    just before, at and just after those edges, and single tokens are
+    decoded across them."""
+    cfg = O.make_cfg([O.attn_layer(heads=4, kv_heads=2, dim=8, vdim=8, softcap=6.0, mlp=None),
+                      O.delta_layer(heads=2, kv_heads=1, dim=8, vdim=8, conv=4, mlp="dense")],
+                     width=12, vocab=19)
+    W, eng = build(cfg, dev, blocks=16, block_size=16)
+    t = toks(196, 19, seed=77)
+    want, _ = O.forward(cfg, W, t)
+    cuts = [15, 1, 1, 46, 1, 1, 63, 1, 1, 2, 64]
+    assert rel_err(run_portions(eng, t, cuts), want) < tol(dev[1])
+
+
 def test_dirty_slot_and_pages_do_not_leak(dev):
     cfg = mixed_cfg()
     W, eng = build(cfg, dev, blocks=6, block_size=4, slots=1)

@@ -3,7 +3,7 @@ docs/ROADMAP.md #4): cached state buffers + wave padding must decode
 identically to the per-wave session path, reuse state across waves, and
 never leak pool blocks (including the padding lanes' scratch block).
 On GPU the same machinery also reuses the captured hipGraph; that
-enablement is a round-2 validation item — here the full state machine
+enablement awaits a GPU validation pass — here the full state machine
 runs on CPU via DISTRL_FORCE_SESSION."""
 
 import pytest
