@@ -623,6 +623,33 @@ def test_checkpoint_registry_and_trace_replay(tmp_path):
     assert rel_err(rd(2), la[8:9]) < 2e-4
 
 
+def test_served_through_the_batcher():
+    """The server's app, batcher and sampler drive the design's engine like
+    any other: greedy completions repeat, sampled ones fan out, logprob
+    rescoring uses the engine's own scoring pass."""
+    from fastapi.testclient import TestClient
+
+    from distrl_llm_amd.serve import create_app
+    from distrl_llm_amd.utils.tokenizer import ByteTokenizer
+    cfg = O.make_cfg([O.attn_layer(heads=4, kv_heads=2, dim=8, vdim=6, mlp="dense"),
+                      O.delta_layer(heads=2, kv_heads=1, dim=8, vdim=6, conv=3, mlp="moe")],
+                     width=16, vocab=600)
+    _, eng = build(cfg, ("cpu", torch.float32), blocks=128, block_size=8, slots=8)
+    client = TestClient(create_app(eng, ByteTokenizer(vocab_size=600), "tiny-nedasun"))
+    body = {"prompt": "2+2=", "max_tokens": 5, "temperature": 0.0}
+    a = client.post("/v1/completions", json=body).json()
+    b = client.post("/v1/completions", json=body).json()
+    assert a["choices"][0]["text"] == b["choices"][0]["text"]
+    assert a["usage"]["completion_tokens"] <= 5
+    r = client.post("/v1/completions", json={"prompt": ["abcd", "wxyz"], "max_tokens": 3,
+                                             "temperature": 1.0, "top_p": 0.9, "n": 2}).json()
+    assert len(r["choices"]) == 4
+    lp = client.post("/v1/completions", json={"prompt": "ab", "max_tokens": 3, "temperature": 0.0,
+                                              "logprobs": 1})
+    assert lp.status_code == 200
+    assert eng.pool.allocator.num_free == 128 and eng.slots.num_free == 8
+
+
 def test_config_errors():
     cfg = mixed_cfg()
     for path, value in [((0, "type"), "other"), ((2, "mixer", "kv_heads"), 4),
