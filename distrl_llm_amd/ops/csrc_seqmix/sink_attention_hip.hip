@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
 // at a time: lane l scores key l, an online softmax carries max and sum
 // across chunks (started at the sink: m = sink, l = 1), then the lanes switch
 // to the value axis and accumulate sum_j p_j v_j over NV = groups * vd dims.
-#define SA_REGS 16   // value dims per lane: groups * vd <= 64 * 16
+#define SA_REGS 32   // value dims per lane: groups * vd <= 64 * 32
 template <typename T>
 __global__ __launch_bounds__(64) void sink_attention_kernel(
     const T* __restrict__ q,          // [Tn, H, dk]

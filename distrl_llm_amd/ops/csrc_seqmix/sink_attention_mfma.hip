@@ -2,9 +2,10 @@
 // up to 64 queries of one head) and decode steps (HEADS: a tile = the heads
 // of one token, the key range split over workgroups and merged afterwards).
 //
-// One workgroup (4 waves) per (tile of <= 64 consecutive queries of one
-// sequence, query head). Wave w owns queries 16 w .. 16 w + 15 for the whole
-// kernel: their scores, their online softmax and their value sums, so the
+// One workgroup (4 waves, or 8 when the value range is wider than 256
+// columns: two sets of 4 that split the columns) per (tile of <= 64
+// consecutive queries of one sequence, query head). Wave w of a set owns
+// queries 16 w .. 16 w + 15 for the whole kernel: their scores, their online softmax and their value sums, so the
 // waves only meet to stage a block of 64 keys: the head's K rows and the V
 // rows (of every kv head when the weights are mixed across heads, of the
 // head's own kv head otherwise) go through LDS once per 64 queries.
@@ -38,8 +39,12 @@ namespace {
 #define SAM_PP 68          // p_lds row pitch (floats): 64 keys + 4
 #define SAM_MAX_KSTEPS 8   // dk <= 256
 
-template <int NT, bool HEADS>   // NT: 16-column value tiles held by a wave (NV <= 16 NT)
-__global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
+// NT: 16-column value tiles held by a wave; WS: wave sets. Set s (waves 4 s ..
+// 4 s + 3) sums value tiles s NT .. s NT + NT - 1 (NV <= 16 NT WS); with two
+// sets both take the scores of the same rows, and the accumulators of a wide
+// value range fit a register budget that lets two waves share a SIMD.
+template <int NT, int WS, bool HEADS>
+__global__ __launch_bounds__(256 * WS, 2) void sink_attention_mfma_kernel(
     const bf16_t* __restrict__ q,         // [Tn, H, dk]
     const bf16_t* __restrict__ cache,     // [rows, G (dk + vd)]
     const int* __restrict__ block_tables, int max_nb, int block_size,
@@ -56,15 +61,18 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
   const int NVp = (NV + 15) / 16 * 16;
   bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem);                 // [64][KP]
   bf16_t* v_lds = k_lds + SAM_KB * KP;                             // [NVp][SAM_VP]
-  float* p_all = reinterpret_cast<float*>(v_lds + NVp * SAM_VP);   // [4][16][SAM_PP]
-  int* krow = reinterpret_cast<int*>(p_all + 4 * 16 * SAM_PP);     // [64]
+  float* p_all = reinterpret_cast<float*>(v_lds + NVp * SAM_VP);   // [4 WS][16][SAM_PP]
+  int* krow = reinterpret_cast<int*>(p_all + 4 * WS * 16 * SAM_PP);   // [64]
+  constexpr int NTH = 256 * WS;
 
   const int tile = blockIdx.x;
   const int hd = HEADS ? 0 : blockIdx.y;
   const int b = HEADS ? tiles[tile] : tiles[3 * tile];
   const int t0 = HEADS ? tile : tiles[3 * tile + 1];
   const int nq = HEADS ? 1 : tiles[3 * tile + 2];
-  const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, lrow = l & 15, lk = l >> 4;
+  const int tid = threadIdx.x, l = tid & 63, lrow = l & 15, lk = l >> 4;
+  const int wave = (tid >> 6) & 3;                 // which 16 rows of the tile
+  const int nt0 = (tid >> 8) * NT;                 // first value tile of the wave's set
   const int W = G * (dk + vd);
   const int rep = H / G;
   const int grp = hd / rep;
@@ -74,7 +82,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
   const int plast = p0 + nq - 1;
   const int nblk = plast / SAM_KB + 1;
   const int* bt = block_tables + (int64_t)b * max_nb;
-  float* p_lds = p_all + wave * 16 * SAM_PP;
+  float* p_lds = p_all + (tid >> 6) * 16 * SAM_PP;
   // uniform per wave: it has rows (queries of the tile, or heads of the token)
   const bool active = HEADS ? (wave * 16 < H) : (wave * 16 < nq);
   const int wave_plast = HEADS ? plast : min(plast, p0 + wave * 16 + 15);
@@ -97,7 +105,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     }
   }
   // padding rows of v_lds (value columns NV .. NVp) stay zero
-  for (int i = tid; i < (NVp - NV) * SAM_VP; i += 256) v_lds[NV * SAM_VP + i] = __float2bfloat16(0.f);
+  for (int i = tid; i < (NVp - NV) * SAM_VP; i += NTH) v_lds[NV * SAM_VP + i] = __float2bfloat16(0.f);
 
   float m[4], lsum[4];
   f32x4 acc[NT];
@@ -115,7 +123,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     }
     __syncthreads();
     // K rows: [key][dk], zero beyond dk
-    if (!HEADS) for (int i = tid; i < SAM_KB * ksteps * 4; i += 256) {
+    if (!HEADS) for (int i = tid; i < SAM_KB * ksteps * 4; i += NTH) {
       const int key = i / (ksteps * 4), c = (i % (ksteps * 4)) * 8;
       bf16v8 v;
       if (c < dk) {
@@ -127,7 +135,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
       *reinterpret_cast<bf16v8*>(k_lds + key * KP + c) = v;
     }
     // V rows, transposed: v_lds[column][key]
-    for (int i = tid; i < SAM_KB * (NV / 8); i += 256) {
+    for (int i = tid; i < SAM_KB * (NV / 8); i += NTH) {
       const int key = i % SAM_KB, c = (i / SAM_KB) * 8;
       const bf16v8 v = *reinterpret_cast<const bf16v8*>(cache + (int64_t)krow[key] * W + voff + c);
       #pragma unroll
@@ -227,14 +235,14 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     }
     #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      if (nt * 16 < NV) {
+      if ((nt0 + nt) * 16 < NV) {
         f32x4 a = acc[nt];
         #pragma unroll
         for (int r = 0; r < 4; ++r) a[r] *= cr[r];
         #pragma unroll
         for (int ks2 = 0; ks2 < 2; ++ks2) {
           const bf16v8 vf = *reinterpret_cast<const bf16v8*>(
-              v_lds + (nt * 16 + lrow) * SAM_VP + ks2 * 32 + lk * 8);
+              v_lds + ((nt0 + nt) * 16 + lrow) * SAM_VP + ks2 * 32 + lk * 8);
           a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi[ks2], vf, a, 0, 0, 0);
           a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo[ks2], vf, a, 0, 0, 0);
         }
@@ -252,13 +260,13 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
       const int head = wave * 16 + lk * 4 + r;
       if (head >= H) continue;
       const int64_t o = ((int64_t)t0 * H + head) * ksplit + blockIdx.y;
-      if (lrow == 0) {
+      if (lrow == 0 && nt0 == 0) {
         part_ml[o * 2] = m[r];
         part_ml[o * 2 + 1] = lsum[r];
       }
       #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const int col = nt * 16 + lrow;
+        const int col = (nt0 + nt) * 16 + lrow;
         if (col < NV) part[o * NV + col] = acc[nt][r];
       }
     }
@@ -279,7 +287,7 @@ __global__ __launch_bounds__(256) void sink_attention_mfma_kernel(
     float* dst = part + ((int64_t)(t0 + qi) * H + hd) * NV;
     #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int col = nt * 16 + lrow;
+      const int col = (nt0 + nt) * 16 + lrow;
       if (col < NV) dst[col] = acc[nt][r] * f;
     }
   }
@@ -313,11 +321,16 @@ __global__ __launch_bounds__(256) void sink_attention_merge_kernel(
   }
 }
 
+// wave sets by value range: one set up to 16 value tiles (two workgroups of
+// four waves then share a CU and overlap their staging and MFMA phases), two
+// beyond; every variant is held to 256 registers so two waves fit a SIMD
+int sam_wave_sets(int NV) { return (NV + 15) / 16 > 16 ? 2 : 1; }
+
 size_t sam_lds_bytes(int dk, int NV, bool heads) {
   const int ksteps = (dk + 31) / 32;
   const int NVp = (NV + 15) / 16 * 16;
   return (heads ? 0 : (size_t)SAM_KB * (ksteps * 32 + 8) * 2) + (size_t)NVp * SAM_VP * 2 +
-         (size_t)4 * 16 * SAM_PP * 4 + SAM_KB * 4;
+         (size_t)4 * sam_wave_sets(NV) * 16 * SAM_PP * 4 + SAM_KB * 4;
 }
 
 }  // namespace
@@ -343,9 +356,9 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
   if (ntiles == 0) return part;
   const size_t lds = sam_lds_bytes(dk, NV, false);
   auto stream = at::cuda::getCurrentCUDAStream();
-#define SAM_LAUNCH(N)                                                                      \
+#define SAM_LAUNCH(N, WSETS)                                                               \
   do {                                                                                     \
-    auto kern = sink_attention_mfma_kernel<N, false>;                                           \
+    auto kern = sink_attention_mfma_kernel<N, WSETS, false>;                                           \
     static int raised = 0;     /* per variant; not repeated under graph capture */         \
     if (lds > 64 * 1024 && (int)lds > raised) {                                            \
       TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                 \
@@ -353,7 +366,7 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
                   "sink attention: cannot raise the LDS limit");                           \
       raised = (int)lds;                                                                   \
     }                                                                                      \
-    kern<<<dim3(ntiles, H), 256, lds, stream>>>(                                           \
+    kern<<<dim3(ntiles, H), 256 * WSETS, lds, stream>>>(                                           \
         reinterpret_cast<const bf16_t*>(q.data_ptr()),                                     \
         reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),   \
         (int)block_tables.size(1), block_size, positions.data_ptr<int>(),                  \
@@ -361,11 +374,11 @@ torch::Tensor sink_attention_mfma(torch::Tensor q, torch::Tensor cache, int H, i
         part.data_ptr<float>(), 1, nullptr);                                               \
   } while (0)
   const int nt = (NV + 15) / 16;
-  if (nt <= 4) SAM_LAUNCH(4);
-  else if (nt <= 8) SAM_LAUNCH(8);
-  else if (nt <= 16) SAM_LAUNCH(16);
-  else if (nt <= 32) SAM_LAUNCH(32);
-  else SAM_LAUNCH(48);
+  if (nt <= 4) SAM_LAUNCH(4, 1);
+  else if (nt <= 8) SAM_LAUNCH(8, 1);
+  else if (nt <= 16) SAM_LAUNCH(16, 1);
+  else if (nt <= 32) SAM_LAUNCH(16, 2);
+  else SAM_LAUNCH(24, 2);
 #undef SAM_LAUNCH
   SM_CHECK_LAUNCH();
   return part;
@@ -390,9 +403,9 @@ torch::Tensor sink_attention_heads(torch::Tensor q, torch::Tensor cache, int H, 
   auto pml = torch::empty({Tn, H, ksplit, 2}, f32);
   const size_t lds = sam_lds_bytes(dk, NV, true);
   auto stream = at::cuda::getCurrentCUDAStream();
-#define SAM_LAUNCH(N)                                                                      \
+#define SAM_LAUNCH(N, WSETS)                                                               \
   do {                                                                                     \
-    auto kern = sink_attention_mfma_kernel<N, true>;                                       \
+    auto kern = sink_attention_mfma_kernel<N, WSETS, true>;                                     \
     static int raised = 0;                                                                 \
     if (lds > 64 * 1024 && (int)lds > raised) {                                            \
       TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                 \
@@ -400,7 +413,7 @@ torch::Tensor sink_attention_heads(torch::Tensor q, torch::Tensor cache, int H, 
                   "sink attention: cannot raise the LDS limit");                           \
       raised = (int)lds;                                                                   \
     }                                                                                      \
-    kern<<<dim3(Tn, ksplit), 256, lds, stream>>>(                                          \
+    kern<<<dim3(Tn, ksplit), 256 * WSETS, lds, stream>>>(                                          \
         reinterpret_cast<const bf16_t*>(q.data_ptr()),                                     \
         reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),   \
         (int)block_tables.size(1), block_size, positions.data_ptr<int>(),                  \
@@ -408,11 +421,11 @@ torch::Tensor sink_attention_heads(torch::Tensor q, torch::Tensor cache, int H, 
         pacc.data_ptr<float>(), ksplit, pml.data_ptr<float>());                            \
   } while (0)
   const int nt = (NV + 15) / 16;
-  if (nt <= 4) SAM_LAUNCH(4);
-  else if (nt <= 8) SAM_LAUNCH(8);
-  else if (nt <= 16) SAM_LAUNCH(16);
-  else if (nt <= 32) SAM_LAUNCH(32);
-  else SAM_LAUNCH(48);
+  if (nt <= 4) SAM_LAUNCH(4, 1);
+  else if (nt <= 8) SAM_LAUNCH(8, 1);
+  else if (nt <= 16) SAM_LAUNCH(16, 1);
+  else if (nt <= 32) SAM_LAUNCH(16, 2);
+  else SAM_LAUNCH(24, 2);
 #undef SAM_LAUNCH
   SM_CHECK_LAUNCH();
   sink_attention_merge_kernel<<<dim3(Tn, H), 256, 0, stream>>>(
