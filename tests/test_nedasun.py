@@ -548,7 +548,9 @@ def test_captured_decode_equals_eager():
                                                  (8, 2, 128, 64, [1, 1, 1, 1], True),
                                                  (4, 4, 32, 64, [1, 1, 1], False),
                                                  (48, 8, 64, 32, [1, 1], True),
-                                                 (6, 3, 40, 24, [1, 1, 1, 1], True)])
+                                                 (6, 3, 40, 24, [1, 1, 1, 1], True),
+                                                 (4, 4, 64, 160, [70, 3], True),
+                                                 (4, 4, 64, 160, [1, 1, 1], True)])
 def test_tiled_attention_kernel_against_plain_op(H, G, dk, vd, lens, talk):
     """bf16 prompt portions take the tiled MFMA kernel, steps of single
     tokens its heads-of-one-token form with split key ranges; the fp32
