@@ -4,7 +4,8 @@
 //                   also / sqrt(dim)), write strength beta = sigmoid(b) and
 //                   decay = exp(-exp(a_log) softplus(a + dt_bias)), all fp32
 //   delta_scan      per (sequence row, head, block of value columns): walks
-//                   the row's tokens in order with the state in registers,
+//                   the row's tokens in order with the state in registers
+//                   (8 key rows of one value column per lane),
 //                   S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
 //                   inputs arrive in chunks through LDS, one chunk ahead
 //   delta_finish    per (token, head): o / rms(o) * norm_w * silu(gate)
@@ -16,7 +17,6 @@
 
 namespace {
 
-#define DR_ROWS 32    // state rows (key dims) held by one lane
 
 // qkv row = [q (G dk) | k (G dk) | v (H vd)] after convolution and SiLU.
 // One workgroup per token; wave w normalises q/k heads w, w + 4, ...
@@ -52,54 +52,79 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
   }
 }
 
-// One wave per (row, head, 64 / KS value columns). Lane = (column, ks): it
-// holds rows ks * 32 .. ks * 32 + 31 of its column; dot products over the key
-// axis are finished with shuffles over the KS lanes of a column. The walk is
-// latency-bound, so the tokens come in chunks of DR_CH: a chunk's unit q/k
-// rows, decays and strengths sit in LDS (every lane reads the same few
-// addresses), the lane's own v entries in registers, and the next chunk is
-// fetched into registers while the current one is walked.
+// One workgroup (4 waves) per (row, head, block of 256 / KS value columns).
+// Lane = (column, ks): it holds DR_ROWS state rows (8 or 32) of its column,
+// starting at ks * DR_ROWS (few rows per lane when there are few sequence
+// rows and heads: the walk is a dependent chain, so it is spread over more
+// lanes and waves rather than made long); dot products over the key axis
+// are finished with lane moves over the KS lanes of a column. The tokens come
+// in chunks of DR_CH: a chunk's unit q/k rows, decays and strengths sit in
+// LDS, shared by the four waves (every lane reads the same few addresses),
+// the lane's own v entries in registers, and the next chunk is fetched into
+// registers while the current one is walked. The state is stored value-major
+// ([head][column][key]): a lane's rows are contiguous and the KS lanes of a
+// column read one contiguous run.
 #define DR_CH 16
-template <typename T, int KS>
-__global__ __launch_bounds__(64) void delta_scan_kernel(
+
+// Sum over the KS adjacent lanes of a column (KS a power of two, groups
+// aligned) with data-parallel lane moves: swaps inside a quad, then a mirror
+// of 8 and of 16 lanes (after the quad steps every lane of a quad holds the
+// quad's sum, so the mirrored lane brings the other half's). These are plain
+// vector instructions; a cross-lane read through LDS per step would put
+// several hundred cycles on the walk's dependent chain.
+template <int CTRL>
+SM_INLINE float dr_lane_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+template <int KS>
+SM_INLINE float dr_column_sum(float x) {
+  if (KS >= 2) x += dr_lane_move<0xB1>(x);     // quad lanes [1, 0, 3, 2]
+  if (KS >= 4) x += dr_lane_move<0x4E>(x);     // quad lanes [2, 3, 0, 1]
+  if (KS >= 8) x += dr_lane_move<0x141>(x);    // mirror within 8 lanes
+  if (KS >= 16) x += dr_lane_move<0x140>(x);   // mirror within 16 lanes
+  if (KS >= 32) x += __shfl_xor(x, 16, SM_WAVE);
+  return x;
+}
+
+template <typename T, int KS, int DR_ROWS>
+__global__ __launch_bounds__(256) void delta_scan_kernel(
     const T* __restrict__ qkv, int C, const float* __restrict__ qn,
     const float* __restrict__ kn, const float* __restrict__ beta,
     const float* __restrict__ decay, float* __restrict__ state,
     const int* __restrict__ cu, const int* __restrict__ slots, int H, int G, int dk,
     int vd, float* __restrict__ o) {
-  constexpr int COLS = 64 / KS;
+  constexpr int COLS = 64 / KS;                 // columns per wave
   constexpr int DKP = KS * DR_ROWS;
   constexpr int ROW4 = DKP / 4;                 // float4 per q or k row
-  constexpr int NPRE = DR_CH * 2 * ROW4 / 64;   // float4 per lane and chunk
+  constexpr int NPRE = DR_CH * 2 * ROW4 / 256;  // float4 per thread and chunk
   __shared__ float4 kq4[DR_CH * 2 * ROW4];      // [token][k | q][DKP]
   __shared__ float sc[DR_CH * 2];               // [token][decay | beta]
   const int b = blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63;
   const int ks = lane % KS;
-  const int col = blockIdx.z * COLS + lane / KS;
+  const int col = (blockIdx.z * 4 + (tid >> 6)) * COLS + lane / KS;
   const int t0 = cu[b], t1 = cu[b + 1];
-  if (t1 == t0) return;
+  if (t1 == t0) return;                         // uniform over the workgroup
   const bool live = col < vd;
   const int g = h / (H / G);
   const int64_t slot = slots[b];
-  float* Sp = state + ((slot * H + h) * dk) * vd + (live ? col : 0);
+  float* Sp = state + ((slot * H + h) * vd + (live ? col : 0)) * dk + ks * DR_ROWS;
   float S[DR_ROWS];
   #pragma unroll
-  for (int r = 0; r < DR_ROWS; ++r) {
-    const int k = ks * DR_ROWS + r;
-    S[r] = (live && k < dk) ? Sp[(int64_t)k * vd] : 0.f;
-  }
+  for (int r = 0; r < DR_ROWS; ++r)
+    S[r] = (live && ks * DR_ROWS + r < dk) ? Sp[r] : 0.f;
   const int voff = 2 * G * dk + h * vd + (live ? col : 0);
 
   float4 pre[NPRE];
   float pv[DR_CH], pvn[DR_CH];
   float psc = 0.f;
   // fetch a chunk into registers: q/k rows (linear float4 index = LDS index),
-  // the lane's v entries, and decay/beta of token lane / 2
+  // the lane's v entries, and decay/beta of token tid / 2
   auto fetch = [&](int tb, int n, float* vout) {
     #pragma unroll
     for (int j = 0; j < NPRE; ++j) {
-      const int i = lane + 64 * j;
+      const int i = tid + 256 * j;
       const int tok = i / (2 * ROW4), rem = i % (2 * ROW4);
       const float* src = (rem >= ROW4 ? qn : kn) + ((int64_t)(tb + min(tok, n - 1)) * G + g) * DKP;
       pre[j] = reinterpret_cast<const float4*>(src)[rem % ROW4];
@@ -107,15 +132,15 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
     #pragma unroll
     for (int i = 0; i < DR_CH; ++i)
       vout[i] = to_f(qkv[(int64_t)(tb + min(i, n - 1)) * C + voff]);
-    if (lane < 2 * DR_CH) {
-      const int64_t t = tb + min(lane >> 1, n - 1);
-      psc = (lane & 1) ? beta[t * H + h] : decay[t * H + h];
+    if (tid < 2 * DR_CH) {
+      const int64_t t = tb + min(tid >> 1, n - 1);
+      psc = (tid & 1) ? beta[t * H + h] : decay[t * H + h];
     }
   };
   auto stash = [&]() {
     #pragma unroll
-    for (int j = 0; j < NPRE; ++j) kq4[lane + 64 * j] = pre[j];
-    if (lane < 2 * DR_CH) sc[lane] = psc;
+    for (int j = 0; j < NPRE; ++j) kq4[tid + 256 * j] = pre[j];
+    if (tid < 2 * DR_CH) sc[tid] = psc;
   };
 
   fetch(t0, min(DR_CH, t1 - t0), pv);
@@ -131,23 +156,20 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
       const float4* kp = kq4 + (i * 2) * ROW4 + ks * (DR_ROWS / 4);
       const float4* qp = kp + ROW4;
       const float dec = sc[2 * i], bt = sc[2 * i + 1];
-      // four partial sums per dot product: no 32-long dependent FMA chain
-      float sk0 = 0.f, sk1 = 0.f, sk2 = 0.f, sk3 = 0.f;
-      float4 kk[DR_ROWS / 4];             // read once: LDS bandwidth bounds the walk
+      float4 kk[DR_ROWS / 4];
+      float sk0 = 0.f, sk1 = 0.f;
       #pragma unroll
       for (int r = 0; r < DR_ROWS; r += 4) {
         const float4 k4 = kk[r / 4] = kp[r / 4];
         S[r] *= dec; S[r + 1] *= dec; S[r + 2] *= dec; S[r + 3] *= dec;
         sk0 = fmaf(S[r], k4.x, sk0);
         sk1 = fmaf(S[r + 1], k4.y, sk1);
-        sk2 = fmaf(S[r + 2], k4.z, sk2);
-        sk3 = fmaf(S[r + 3], k4.w, sk3);
+        sk0 = fmaf(S[r + 2], k4.z, sk0);
+        sk1 = fmaf(S[r + 3], k4.w, sk1);
       }
-      float sk = (sk0 + sk1) + (sk2 + sk3);
-      #pragma unroll
-      for (int off = 1; off < KS; off <<= 1) sk += __shfl_xor(sk, off, SM_WAVE);
+      const float sk = dr_column_sum<KS>(sk0 + sk1);
       const float u = bt * (pv[i] - sk);
-      float so0 = 0.f, so1 = 0.f, so2 = 0.f, so3 = 0.f;
+      float so0 = 0.f, so1 = 0.f;
       #pragma unroll
       for (int r = 0; r < DR_ROWS; r += 4) {
         const float4 k4 = kk[r / 4];
@@ -158,12 +180,10 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
         S[r + 3] = fmaf(k4.w, u, S[r + 3]);
         so0 = fmaf(S[r], q4.x, so0);
         so1 = fmaf(S[r + 1], q4.y, so1);
-        so2 = fmaf(S[r + 2], q4.z, so2);
-        so3 = fmaf(S[r + 3], q4.w, so3);
+        so0 = fmaf(S[r + 2], q4.z, so0);
+        so1 = fmaf(S[r + 3], q4.w, so1);
       }
-      float so = (so0 + so1) + (so2 + so3);
-      #pragma unroll
-      for (int off = 1; off < KS; off <<= 1) so += __shfl_xor(so, off, SM_WAVE);
+      const float so = dr_column_sum<KS>(so0 + so1);
       if (live && ks == 0) o[((int64_t)(tb + i) * H + h) * vd + col] = so;
     }
     __syncthreads();
@@ -175,10 +195,8 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(
     __syncthreads();
   }
   #pragma unroll
-  for (int r = 0; r < DR_ROWS; ++r) {
-    const int k = ks * DR_ROWS + r;
-    if (live && k < dk) Sp[(int64_t)k * vd] = S[r];
-  }
+  for (int r = 0; r < DR_ROWS; ++r)
+    if (live && ks * DR_ROWS + r < dk) Sp[r] = S[r];
 }
 
 // One wave per (token, head).
@@ -200,19 +218,19 @@ __global__ __launch_bounds__(64) void delta_finish_kernel(
 }
 
 template <typename T>
-void launch_scan(int KS, dim3 grid, hipStream_t stream, const T* qkv, int C, const float* qn,
+void launch_scan(int KS, int R, dim3 grid, hipStream_t stream, const T* qkv, int C, const float* qn,
                  const float* kn, const float* beta, const float* decay, float* state,
                  const int* cu, const int* slots, int H, int G, int dk, int vd, float* o) {
-#define DR_CASE(N)                                                                       \
-  case N:                                                                                \
-    delta_scan_kernel<T, N><<<dim3(grid.x, grid.y, SM_CDIV(vd, 64 / N)), 64, 0, stream>>>( \
-        qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, vd, o);                 \
-    break;
-  switch (KS) {
-    DR_CASE(1) DR_CASE(2) DR_CASE(4) DR_CASE(8)
-    default: TORCH_CHECK(false, "gated_delta_rule: key dim too large");
+#define DR_CASE(N, RR)                                                                        \
+  if (KS == N && R == RR) {                                                                   \
+    delta_scan_kernel<T, N, RR><<<dim3(grid.x, grid.y, SM_CDIV(vd, 256 / N)), 256, 0, stream>>>( \
+        qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, vd, o);                      \
+    return;                                                                                   \
   }
+  DR_CASE(4, 8) DR_CASE(8, 8) DR_CASE(16, 8) DR_CASE(32, 8)
+  DR_CASE(1, 32) DR_CASE(2, 32) DR_CASE(4, 32) DR_CASE(8, 32)
 #undef DR_CASE
+  TORCH_CHECK(false, "gated_delta_rule: key dim too large");
 }
 
 }  // namespace
@@ -238,10 +256,15 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
   TORCH_CHECK(a_log.numel() == H && dt_bias.numel() == H && onorm_w.numel() == vd, "gated_delta_rule: per-head tensors");
   TORCH_CHECK(state.dim() == 2 && state.size(1) == (int64_t)H * dk * vd && cu.numel() == B + 1,
               "gated_delta_rule: state/batch layout");
-  int KS = 1;
-  while (KS * DR_ROWS < dk) KS *= 2;
-  TORCH_CHECK(KS <= 8, "gated_delta_rule: key dim above 256");
-  const int dkp = KS * DR_ROWS;
+  TORCH_CHECK(dk <= 256, "gated_delta_rule: key dim above 256");
+  int dkp = 32;
+  while (dkp < dk) dkp *= 2;
+  // 32 state rows per lane once that gives every SIMD of the chip a wave
+  // (fewer lane moves and LDS reads per multiply-add); 8 rows, four times the
+  // lanes, below that (measured crossover on 256 CUs: 1024 waves)
+  const int64_t waves32 = (int64_t)B * H * SM_CDIV(vd * (dkp / 32), 64);
+  const int R = waves32 >= 1024 ? 32 : 8;
+  const int KS = dkp / R;
   auto out = torch::empty({T, (int64_t)H * vd}, qkv.options());
   if (T == 0 || B == 0) return out;
   auto f32 = qkv.options().dtype(at::kFloat);
@@ -258,7 +281,7 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
         xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
-    launch_scan<bf16_t>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+    launch_scan<bf16_t>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                         beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
                         cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();
@@ -271,7 +294,7 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
         xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
-    launch_scan<float>(KS, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+    launch_scan<float>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                        beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();

@@ -303,7 +303,7 @@ def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
     beta = sigmoid(b); decay = exp(-exp(a_log) softplus(a + dt_bias));
     S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
     out = o / rms(o) * onorm_w * silu(gate). state fp32
-    [slots, H * dim * vdim], advanced in place."""
+    [slots, H * vdim * dim] (per head value-major: S^T), advanced in place."""
     T = qkv.shape[0]
     H, G = heads, kv_heads
     rep = H // G
@@ -321,13 +321,13 @@ def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
     o = torch.empty(T, H, vdim, dtype=torch.float32, device=qkv.device)
     cu_l, slots_l = cu.tolist(), slots.tolist()
     for b, s in enumerate(slots_l):
-        S = state[s].view(H, dim, vdim).clone()
+        S = state[s].view(H, vdim, dim).transpose(1, 2).clone()
         for t in range(cu_l[b], cu_l[b + 1]):
             S = decay[t][:, None, None] * S
             u = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
             S = S + k[t][:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hkv,hk->hv", S, q[t])
-        state[s] = S.reshape(-1)
+        state[s] = S.transpose(1, 2).reshape(-1)
     o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * onorm_w.float()
     g = gate.float().view(T, H, vdim)
     return (o * g * torch.sigmoid(g)).reshape(T, H * vdim).to(out_dtype)
