@@ -110,10 +110,20 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   const int g = h / (H / G);
   const int64_t slot = slots[b];
   float* Sp = state + ((slot * H + h) * vd + (live ? col : 0)) * dk + ks * DR_ROWS;
+  const bool vec = (dk % 4) == 0;               // a lane's rows as 16-byte pieces
   float S[DR_ROWS];
   #pragma unroll
-  for (int r = 0; r < DR_ROWS; ++r)
-    S[r] = (live && ks * DR_ROWS + r < dk) ? Sp[r] : 0.f;
+  for (int r = 0; r < DR_ROWS; r += 4) {
+    const int k = ks * DR_ROWS + r;
+    if (vec) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (live && k < dk) v = *reinterpret_cast<const float4*>(Sp + r);
+      S[r] = v.x; S[r + 1] = v.y; S[r + 2] = v.z; S[r + 3] = v.w;
+    } else {
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) S[r + j] = (live && k + j < dk) ? Sp[r + j] : 0.f;
+    }
+  }
   const int voff = 2 * G * dk + h * vd + (live ? col : 0);
 
   float4 pre[NPRE];
@@ -195,8 +205,17 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     __syncthreads();
   }
   #pragma unroll
-  for (int r = 0; r < DR_ROWS; ++r)
-    if (live && ks * DR_ROWS + r < dk) Sp[r] = S[r];
+  for (int r = 0; r < DR_ROWS; r += 4) {
+    const int k = ks * DR_ROWS + r;
+    if (vec) {
+      if (live && k < dk)
+        *reinterpret_cast<float4*>(Sp + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+      #pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (live && k + j < dk) Sp[r + j] = S[r + j];
+    }
+  }
 }
 
 // One wave per (token, head).
@@ -261,9 +280,12 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
   while (dkp < dk) dkp *= 2;
   // 32 state rows per lane once that gives every SIMD of the chip a wave
   // (fewer lane moves and LDS reads per multiply-add); 8 rows, four times the
-  // lanes, below that (measured crossover on 256 CUs: 1024 waves)
+  // lanes, below that
+  // (measured crossover on 256 CUs: 1024 waves). Steps of a few tokens per
+  // row are bound by reading and writing the state: 8 rows per lane make the
+  // KS lanes of a column one contiguous run of 16-byte pieces.
   const int64_t waves32 = (int64_t)B * H * SM_CDIV(vd * (dkp / 32), 64);
-  const int R = waves32 >= 1024 ? 32 : 8;
+  const int R = (waves32 >= 1024 && T >= 8 * (int64_t)B) ? 32 : 8;
   const int KS = dkp / R;
   auto out = torch::empty({T, (int64_t)H * vd}, qkv.options());
   if (T == 0 || B == 0) return out;

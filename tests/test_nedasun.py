@@ -308,23 +308,23 @@ def test_delta_rule_against_oracle(dev, H, G, dk, vd):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,H,G,dk,vd", [(32, 32, 8, 32, 64), (16, 16, 4, 72, 40)])
 def test_delta_rule_many_rows_layout(dtype, B, H, G, dk, vd):
-    """With many rows and heads the scan keeps 32 state rows per lane
-    instead of 8; the torch form of the op (itself held to the oracle on
-    the CPU) must agree, two steps in a row so that the stored state is
-    read back."""
+    """With many rows and heads and several tokens per row the scan keeps
+    32 state rows per lane instead of 8; the torch form of the op (itself
+    held to the oracle on the CPU) must agree, two steps in a row so that
+    the stored state is read back (the second by the 8-row form)."""
     from distrl_llm_amd.ops import seqmix_reference as R
     g = torch.Generator().manual_seed(11)
-    lens = [1 + (i % 3) for i in range(B)]
-    T, C = sum(lens), 2 * G * dk + H * vd
-    cu = [0]
-    for n in lens:
-        cu.append(cu[-1] + n)
+    C = 2 * G * dk + H * vd
     a_log, dtb = 0.5 * torch.randn(H, generator=g), 0.5 * torch.randn(H, generator=g)
     nw = 1.0 + 0.1 * torch.randn(vd, generator=g)
     st_cpu = torch.zeros(B + 1, H * dk * vd)
     st_gpu = st_cpu.clone().cuda()
     slots = torch.randperm(B + 1, generator=g)[:B].to(torch.int32)
     for step in range(2):
+        lens = [(9 if step == 0 else 1) + (i % 3) for i in range(B)]
+        T, cu = sum(lens), [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
         qkv = torch.randn(T, C, generator=g).to(dtype)
         gate = torch.randn(T, H * vd, generator=g).to(dtype)
         ab = torch.randn(T, 2 * H, generator=g)
