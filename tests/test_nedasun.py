@@ -266,7 +266,7 @@ def test_conv_silu_portions(dev, taps):
 @pytest.mark.parametrize("H,G,dk,vd", [(4, 2, 8, 6), (2, 1, 40, 5), (3, 3, 5, 70), (2, 2, 72, 9)])
 def test_delta_rule_against_oracle(dev, H, G, dk, vd):
     """The recurrence alone: identity projections turn the oracle's mixer
-    into the op's contract. Portions and a second row share the steps."""
+    into the op's inputs. Portions and a second row share the steps."""
     device, dtype = dev
     n, eps = 19, 1e-5
     g = torch.Generator().manual_seed(5)
