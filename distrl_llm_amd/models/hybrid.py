@@ -665,7 +665,22 @@ def load_nedasun_checkpoint(path: str, dtype=torch.bfloat16, device=None) -> Hyb
         cfg = json.load(f)
     name = os.path.basename(os.path.normpath(path)) or "nedasun"
     model = HybridLM(nedasun_spec_from_config(cfg, name), dtype=dtype, device=device)
-    model.load_tensors(load_file(os.path.join(path, "model.safetensors")))
+    tensors = load_file(os.path.join(path, "model.safetensors"))
+    known = model._named_slices()
+    extra = sorted(k for k in tensors if k not in known)
+    if extra:
+        import sys
+        sys.stderr.write(f"[nedasun] ignoring {len(extra)} tensors the design "
+                         f"does not name: {extra[:4]}\n")
+    # the blend factor is read only by mixing layers after the first one: a
+    # checkpoint may leave it out elsewhere
+    unused = {f"l{i}.mix.vmix" for i, ls in enumerate(model.spec.layers)
+              if isinstance(ls.mixer, SinkAttentionSpec) and ls.mixer.v_first is None}
+    have = {k: v for k, v in tensors.items() if k in known}
+    missing = set(known) - set(have) - unused
+    if missing:
+        raise ValueError(f"checkpoint misses tensors: {sorted(missing)[:8]}")
+    model.load_tensors(have, strict=False)
     return model
 
 

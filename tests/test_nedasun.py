@@ -633,9 +633,23 @@ def test_checkpoint_registry_and_trace_replay(tmp_path):
     from safetensors.torch import load_file
     back = load_file(os.path.join(ck, "model.safetensors"))
     assert set(back) == set(W) and back["l2.mix.vmix"].shape == ()
+    # the blend factor of layers that never read it may be left out; a tensor
+    # the design does not name is ignored; anything else missing is an error
+    from safetensors.torch import save_file
+    trimmed = {k: v for k, v in back.items() if k not in ("l0.mix.vmix", "l2.mix.vmix")}
+    trimmed["l0.mix.other"] = torch.zeros(3)
+    save_file(trimmed, os.path.join(ck, "model.safetensors"))
     m2, eng = load_model_and_engine(ck, EngineConfig(num_kv_blocks=8, num_state_slots=2),
                                     dtype=torch.float32, device=torch.device("cpu"))
     assert isinstance(eng, HybridEngine) and m2.spec.block == "sandwich"
+    bad = str(tmp_path / "bad")
+    os.makedirs(bad)
+    save_file({k: v for k, v in back.items() if k != "l4.mix.vmix"},
+              os.path.join(bad, "model.safetensors"))
+    json.dump(saved, open(os.path.join(bad, "config.json"), "w"))
+    with pytest.raises(ValueError):
+        load_model_and_engine(bad, EngineConfig(num_kv_blocks=8, num_state_slots=2),
+                              dtype=torch.float32, device=torch.device("cpu"))
     a, b = toks(9, cfg["vocab"], seed=50), toks(5, cfg["vocab"], seed=51)
     steps = [{"step": 0, "entries": [{"id": "x", "tokens": a[:4], "want": [3]}], "end": []},
              {"step": 1, "entries": [{"id": "x", "tokens": a[4:8], "want": []},
