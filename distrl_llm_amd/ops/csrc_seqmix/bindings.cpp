@@ -60,8 +60,10 @@ torch::Tensor sink_attention(torch::Tensor q, torch::Tensor cache, int64_t heads
                              double softcap, c10::optional<torch::Tensor> sink,
                              c10::optional<torch::Tensor> talk,
                              c10::optional<torch::Tensor> tiles, int64_t max_tile_queries);
-torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Tensor ab,
-                               torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
+torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
+                               c10::optional<torch::Tensor> ab,
+                               c10::optional<torch::Tensor> h,
+                               c10::optional<torch::Tensor> ab_w, torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
                                double eps, torch::Tensor state, torch::Tensor cu,
                                torch::Tensor slots, int64_t heads, int64_t kv_heads,
                                int64_t dim, int64_t vdim);

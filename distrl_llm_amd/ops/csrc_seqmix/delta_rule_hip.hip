@@ -3,7 +3,8 @@
 // head). Three kernels:
 //   delta_prepare   per token: q, k of every q/k head made unit vectors (q
 //                   also / sqrt(dim)), write strength beta = sigmoid(b) and
-//                   decay = exp(-exp(a_log) softplus(a + dt_bias)), all fp32
+//                   decay = exp(-exp(a_log) softplus(a + dt_bias)), all fp32;
+//                   b and a are given, or projected here from the mixer input
 //   delta_scan      per (sequence row, head, block of value columns): walks
 //                   the row's tokens in order with the state in registers
 //                   (8 key rows of one value column per lane),
@@ -24,12 +25,38 @@ namespace {
 template <typename T>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const T* __restrict__ qkv, int C, const float* __restrict__ ab,
+    const T* __restrict__ hin, int64_t ldh, const float* __restrict__ ab_w, int D,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, int H, int G,
     int dk, int dkp, float* __restrict__ qn, float* __restrict__ kn,
     float* __restrict__ beta, float* __restrict__ decay) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = qkv + t * C;
+  if (blockIdx.y > 0) {
+    // the [strength; step] projection of the mixer input, fp32: one wave per
+    // output, four outputs per workgroup (blockIdx.y - 1 counts the groups)
+    const int j = (blockIdx.y - 1) * 4 + wave;
+    if (j >= 2 * H) return;
+    const float* wr = ab_w + (int64_t)j * D;
+    float a0 = 0.f, a1 = 0.f;
+    int d = lane;
+    for (; d + 64 < D; d += 128) {
+      a0 = fmaf(to_f(hin[t * ldh + d]), wr[d], a0);
+      a1 = fmaf(to_f(hin[t * ldh + d + 64]), wr[d + 64], a1);
+    }
+    if (d < D) a0 = fmaf(to_f(hin[t * ldh + d]), wr[d], a0);
+    const float z = sm_wave_sum(a0 + a1);
+    if (lane == 0) {
+      if (j < H) {
+        beta[t * H + j] = sm_sigmoid(z);
+      } else {
+        const float y = z + dt_bias[j - H];
+        const float sp = (y > 20.f) ? y : log1pf(expf(y));
+        decay[t * H + j - H] = expf(-expf(a_log[j - H]) * sp);
+      }
+    }
+    return;
+  }
   for (int job = wave; job < 2 * G; job += 4) {
     const bool is_k = job >= G;
     const int g = is_k ? job - G : job;
@@ -45,7 +72,7 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
     float* dst = (is_k ? kn : qn) + (t * G + g) * dkp;
     for (int k = lane; k < dkp; k += 64) dst[k] = (k < dk) ? to_f(src[k]) * inv : 0.f;
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+  if (ab != nullptr) for (int h = threadIdx.x; h < H; h += blockDim.x) {
     beta[t * H + h] = sm_sigmoid(ab[t * 2 * H + h]);
     const float z = ab[t * 2 * H + H + h] + dt_bias[h];
     const float sp = (z > 20.f) ? z : log1pf(expf(z));
@@ -255,12 +282,15 @@ void launch_scan(int KS, int R, dim3 grid, hipStream_t stream, const T* qkv, int
 
 }  // namespace
 
-torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Tensor ab,
+torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
+                               c10::optional<torch::Tensor> ab_opt,
+                               c10::optional<torch::Tensor> h_opt,
+                               c10::optional<torch::Tensor> ab_w_opt,
                                torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
                                double eps, torch::Tensor state, torch::Tensor cu,
                                torch::Tensor slots, int64_t heads, int64_t kv_heads,
                                int64_t dim, int64_t vdim) {
-  SM_CHECK_CUDA(qkv); SM_CHECK_CUDA(ab); SM_CHECK_F32(ab);
+  SM_CHECK_CUDA(qkv);
   SM_CHECK_CUDA(a_log); SM_CHECK_F32(a_log); SM_CHECK_CUDA(dt_bias); SM_CHECK_F32(dt_bias);
   SM_CHECK_CUDA(onorm_w); SM_CHECK_F32(onorm_w); SM_CHECK_CUDA(state); SM_CHECK_F32(state);
   SM_CHECK_CUDA(cu); SM_CHECK_I32(cu); SM_CHECK_CUDA(slots); SM_CHECK_I32(slots);
@@ -272,7 +302,31 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
   TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == C, "gated_delta_rule: qkv width");
   TORCH_CHECK(gate.is_cuda() && gate.dim() == 2 && gate.stride(1) == 1 && gate.size(0) == T &&
               gate.size(1) == H * vd && gate.scalar_type() == qkv.scalar_type(), "gated_delta_rule: gate layout");
-  TORCH_CHECK(ab.dim() == 2 && ab.size(0) == T && ab.size(1) == 2 * H, "gated_delta_rule: ab is [T, 2H]");
+  // the write strength / step inputs: given as [T, 2H] fp32, or computed here
+  // from the mixer input h [T, D] and the fp32 matrix ab_w [2H, D]
+  const float* abp = nullptr;
+  const float* abwp = nullptr;
+  const void* hp = nullptr;
+  int64_t ldh = 0;
+  int Dh = 0;
+  if (ab_opt.has_value()) {
+    const torch::Tensor& ab = *ab_opt;
+    SM_CHECK_CUDA(ab); SM_CHECK_F32(ab);
+    TORCH_CHECK(ab.dim() == 2 && ab.size(0) == T && ab.size(1) == 2 * H, "gated_delta_rule: ab is [T, 2H]");
+    abp = ab.data_ptr<float>();
+  } else {
+    TORCH_CHECK(h_opt.has_value() && ab_w_opt.has_value(), "gated_delta_rule: ab, or h with ab_w");
+    const torch::Tensor& hh = *h_opt;
+    const torch::Tensor& w = *ab_w_opt;
+    SM_CHECK_CUDA(w); SM_CHECK_F32(w);
+    TORCH_CHECK(hh.is_cuda() && hh.dim() == 2 && hh.stride(1) == 1 && hh.size(0) == T &&
+                hh.scalar_type() == qkv.scalar_type(), "gated_delta_rule: h layout");
+    TORCH_CHECK(w.dim() == 2 && w.size(0) == 2 * H && w.size(1) == hh.size(1), "gated_delta_rule: ab_w is [2H, D]");
+    hp = hh.data_ptr();
+    ldh = hh.stride(0);
+    Dh = hh.size(1);
+    abwp = w.data_ptr<float>();
+  }
   TORCH_CHECK(a_log.numel() == H && dt_bias.numel() == H && onorm_w.numel() == vd, "gated_delta_rule: per-head tensors");
   TORCH_CHECK(state.dim() == 2 && state.size(1) == (int64_t)H * dk * vd && cu.numel() == B + 1,
               "gated_delta_rule: state/batch layout");
@@ -298,10 +352,12 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
   const bool bf16 = qkv.scalar_type() == at::kBFloat16;
   if (!bf16) SM_CHECK_F32(qkv);
   dim3 gscan(B, H), gfin(T, H);
+  dim3 gprep(T, abp != nullptr ? 1 : 1 + SM_CDIV(2 * H, 4));
   if (bf16) {
     const bf16_t* xp = reinterpret_cast<const bf16_t*>(qkv.data_ptr());
-   hipLaunchKernelGGL(( delta_prepare_kernel<bf16_t>), dim3(T), dim3(256), 0, stream, 
-        xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
+   hipLaunchKernelGGL(( delta_prepare_kernel<bf16_t>), dim3(gprep), dim3(256), 0, stream, 
+        xp, C, abp, reinterpret_cast<const bf16_t*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
+        dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
     launch_scan<bf16_t>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
@@ -313,8 +369,9 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate, torch::Ten
         onorm_w.data_ptr<float>(), (float)eps, H, vd, reinterpret_cast<bf16_t*>(out.data_ptr()));
   } else {
     const float* xp = qkv.data_ptr<float>();
-   hipLaunchKernelGGL(( delta_prepare_kernel<float>), dim3(T), dim3(256), 0, stream, 
-        xp, C, ab.data_ptr<float>(), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), H, G, dk, dkp,
+   hipLaunchKernelGGL(( delta_prepare_kernel<float>), dim3(gprep), dim3(256), 0, stream, 
+        xp, C, abp, reinterpret_cast<const float*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
+        dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
     launch_scan<float>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),

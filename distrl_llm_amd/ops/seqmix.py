@@ -197,11 +197,16 @@ def tap_conv_silu(x, w, tails, cu, tok_seq, slots, out_dtype):
 
 
 def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
-                     slots, heads, kv_heads, dim, vdim, out_dtype):
+                     slots, heads, kv_heads, dim, vdim, out_dtype, h=None,
+                     ab_w=None):
+    """``ab`` None: the [strength | step] inputs are projected inside the op
+    from the mixer input ``h`` with the fp32 matrix ``ab_w`` [2H, D]."""
     if qkv.is_cuda:
         return _ext("gated_delta_rule").gated_delta_rule(
-            qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu, slots,
-            heads, kv_heads, dim, vdim)
+            qkv, gate, ab, h, ab_w, a_log, dt_bias, onorm_w, eps, state, cu,
+            slots, heads, kv_heads, dim, vdim)
+    if ab is None:
+        ab = torch.nn.functional.linear(h.float(), ab_w.float())
     return R.gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps,
                               state, cu, slots, heads, kv_heads, dim, vdim,
                               out_dtype)
