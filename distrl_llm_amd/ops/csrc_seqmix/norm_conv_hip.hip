@@ -117,6 +117,31 @@ __global__ __launch_bounds__(256) void tap_tail_kernel(
     if (k < keep) tails[(slot * keep + k) * D + d] = nv[k];
 }
 
+// Steps in which every row brings one token: conv and tail update in one
+// kernel, one thread per (row, channel) (it alone touches that tail).
+template <typename Tin, typename T, bool ADD_IN, bool SILU>
+__global__ __launch_bounds__(256) void tap_conv_step_kernel(
+    const Tin* __restrict__ h, int64_t ld, const float* __restrict__ w,
+    float* __restrict__ tails, const int* __restrict__ slots, int D, int taps,
+    T* __restrict__ out) {
+  const int b = blockIdx.x;
+  const int d = blockIdx.y * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  const int keep = taps - 1;
+  float* tl = tails + (int64_t)slots[b] * keep * D + d;
+  const float x = to_f(h[(int64_t)b * ld + d]);
+  float acc = (ADD_IN ? x : 0.f) + w[d * taps + keep] * x;
+  float prev = x;                       // becomes the newest tail entry
+  for (int j = keep - 1; j >= 0; --j) {
+    const float v = tl[(int64_t)j * D];
+    acc += w[d * taps + j] * v;
+    tl[(int64_t)j * D] = prev;          // shift: entry j takes what entry j + 1 held
+    prev = v;
+  }
+  if (SILU) acc = acc * sm_sigmoid(acc);
+  out[(int64_t)b * D + d] = from_f<T>(acc);
+}
+
 // x += s / sqrt(mean(s^2) + eps) * (1 + post_w), s = y (+ y2); then, with
 // next_w, h = x / sqrt(mean(x^2) + eps) * (1 + next_w). y and y2 are bf16 or
 // fp32 each (flags), h is T.
@@ -315,6 +340,20 @@ torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tail
   if (T == 0) return out;
   auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA();
   dim3 grid(T, SM_CDIV(C, 256)), g2(B, SM_CDIV(C, 256));
+  if (T == B) {
+    // one token per row (cu is 0, 1, 2, ...: a step's rows are never empty)
+    if (in_bf16)
+     hipLaunchKernelGGL(( tap_conv_step_kernel<bf16_t, bf16_t, false, true>), dim3(g2), dim3(256), 0, stream, 
+          reinterpret_cast<const bf16_t*>(x.data_ptr()), ld, w.data_ptr<float>(),
+          tails.data_ptr<float>(), slots.data_ptr<int>(), C, taps,
+          reinterpret_cast<bf16_t*>(out.data_ptr()));
+    else
+     hipLaunchKernelGGL(( tap_conv_step_kernel<float, float, false, true>), dim3(g2), dim3(256), 0, stream, 
+          x.data_ptr<float>(), ld, w.data_ptr<float>(), tails.data_ptr<float>(),
+          slots.data_ptr<int>(), C, taps, out.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+    return out;
+  }
   if (in_bf16) {
     const bf16_t* xp = reinterpret_cast<const bf16_t*>(x.data_ptr());
    hipLaunchKernelGGL(( tap_conv_kernel<bf16_t, bf16_t, false, true>), dim3(grid), dim3(256), 0, stream, 

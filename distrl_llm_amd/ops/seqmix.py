@@ -189,7 +189,9 @@ def sink_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
 
 
 def tap_conv_silu(x, w, tails, cu, tok_seq, slots, out_dtype):
-    """``x`` may be a column slice of a wider row-major matrix."""
+    """``x`` may be a column slice of a wider row-major matrix. Every row of
+    the step holds at least one token (a step whose rows all hold exactly
+    one runs conv and tail update as one kernel)."""
     if x.is_cuda:
         return _ext("tap_conv_silu").tap_conv_silu(x, w, tails, cu, tok_seq,
                                                    slots, _bf16(out_dtype))
