@@ -362,12 +362,17 @@ class HybridEngine:
         qkv = SM.tap_conv_silu(proj[:, :C], L.conv_w, self.slots.mixer_tails[i],
                                meta["cu"], meta["tok_seq"], meta["slots"],
                                self.dtype)
-        # the decay / strength inputs are projected in fp32 inside the op
-        o = SM.gated_delta_rule(qkv, proj[:, C:], None, L.a_log, L.dt_bias,
+        # fp32 decay / strength inputs: a GEMM for prompt-sized steps; steps
+        # of a few tokens project them inside the op (two launches fewer)
+        if hm.shape[0] <= 256:
+            ab, own = None, dict(h=hm, ab_w=L.ab_w)
+        else:
+            ab, own = F.linear(hm.float(), L.ab_w), {}
+        o = SM.gated_delta_rule(qkv, proj[:, C:], ab, L.a_log, L.dt_bias,
                                 L.onorm_w, self.spec.norm_eps,
                                 self.slots.recurrent[i], meta["cu"],
                                 meta["slots"], m.heads, m.kv_heads, m.dim,
-                                m.vdim, self.dtype, h=hm, ab_w=L.ab_w)
+                                m.vdim, self.dtype, **own)
         return F.linear(o, L.out_w)
 
     def _mixer(self, i, ls, L, hm, meta, shared):
